@@ -1,6 +1,6 @@
 """Device tensors of the cache: for every run of the model's order that keeps keys and
 values, K [pages, kv_heads, page, head_dim] and V [pages, kv_heads, page / vt, head_dim, vt]
-of its group's page count; for every run with fixed state, its tensors [slots + 1, ...] (the
+(head_dim the values' own size where the run's need names one) of its group's page count; for every run with fixed state, its tensors [slots + 1, ...] (the
 last row belongs to no request: rows that pad a captured batch read and write it).
 
 Reference: nanovllm/engine/model_runner.py:103-121 keeps one tensor [2, layers, pages,
@@ -20,8 +20,13 @@ from ..parts.model import LayerCache, torch_dtype
 
 def bytes_per_page(needs, groups, page_size: int, itemsize: int) -> List[int]:
     """Per group: bytes that one page takes over all the group's runs."""
-    return [sum(2 * needs[r].num_kv_heads * needs[r].head_dim * page_size * itemsize for r in g.runs)
-            for g in groups]
+    return [sum(needs[r].num_kv_heads * (needs[r].head_dim + _value_dim(needs[r])) * page_size * itemsize
+                for r in g.runs) for g in groups]
+
+
+def _value_dim(need) -> int:
+    v = getattr(need, "v_head_dim", None)
+    return need.head_dim if v is None else v
 
 
 def state_bytes_per_slot(needs, state_runs) -> int:
@@ -46,7 +51,7 @@ def allocate(needs, groups, state_runs, num_pages: Sequence[int], page_size: int
         for r in group.runs:
             need = needs[r]
             k = torch.zeros((num_pages[g], need.num_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
-            v = torch.zeros(v_cache_shape(num_pages[g], need.num_kv_heads, need.head_dim, page_size), dtype=dtype,
+            v = torch.zeros(v_cache_shape(num_pages[g], need.num_kv_heads, _value_dim(need), page_size), dtype=dtype,
                             device=device)
             caches[r] = LayerCache(group=g, k=k, v=v)
     for r in state_runs:

@@ -171,3 +171,154 @@ def read_config_json(folder: str) -> dict:
         raise ConfigError(f"{folder!r} holds no config.json")
     with open(path) as f:
         return json.load(f)
+
+
+# ---------------------------------------------------------------------------- Nozurax
+def _section(d: Mapping[str, Any], key: str, where: str) -> Mapping[str, Any]:
+    v = d.get(key)
+    if not isinstance(v, Mapping):
+        raise ConfigError(f"{where}: key {key!r} must be an object")
+    return v
+
+
+@dataclass(frozen=True)
+class NozuraxLayer:
+    """One entry of config.json's "layers".  kind: "attention" | "retention".  weights_of: the
+    entry whose tensors this one runs (itself where it has its own).  ff: the feed-forward's inner
+    size, None for a layer without one.  The mixer's sizes and constants by their config names:
+    attention  heads, kv_heads, dim, vdim, scale, temp_coef, temp_every (temp_coef 0: no temperature)
+    retention  heads, dim, vdim, decay (one per head), rot_dims, rot_base (rot_dims 0: no rotation)"""
+    kind: str
+    weights_of: int
+    ff: Optional[int]
+    heads: int
+    dim: int
+    vdim: int
+    kv_heads: int = 0
+    scale: float = 1.0
+    temp_coef: float = 0.0
+    temp_every: int = 1
+    decay: Tuple[float, ...] = ()
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+
+
+@dataclass(frozen=True)
+class NozuraxConfig:
+    """Nozurax: a decoder whose layers add a mixer and a feed-forward that read the same norm, with
+    retention and sink-attention mixers in an order the configuration gives, and layers that may run
+    another layer's tensors again.  config.json gives every size and constant."""
+    vocab: int
+    width: int
+    eps: float
+    layers: Tuple[NozuraxLayer, ...]
+    dtype: str = "bfloat16"
+    eos_token_id: Optional[Tuple[int, ...]] = None
+    architecture: str = "Nozurax"
+
+    @classmethod
+    def from_dict(cls, d: Mapping[str, Any]) -> "NozuraxConfig":
+        where = "config.json"
+        entries = d.get("layers")
+        if not isinstance(entries, (list, tuple)):
+            raise ConfigError(f"{where}: key 'layers' must be a list")
+        layers = []
+        for i, entry in enumerate(entries):
+            at = f"{where}: layers[{i}]"
+            if not isinstance(entry, Mapping):
+                raise ConfigError(f"{at} must be an object")
+            kind = entry.get("type")
+            m = _section(entry, "mixer", at)
+            mlp = entry.get("mlp")
+            ff = None
+            if mlp is not None:
+                if not isinstance(mlp, Mapping) or mlp.get("kind", "dense") != "dense":
+                    raise ConfigError(f"{at}: mlp must be null or an object of kind 'dense', got {mlp!r}")
+                ff = _require(mlp, "ff", int, at + ".mlp")
+            common = dict(kind=kind, weights_of=int(entry.get("weights_of", i)), ff=ff,
+                          heads=_require(m, "heads", int, at + ".mixer"), dim=_require(m, "dim", int, at + ".mixer"),
+                          vdim=_require(m, "vdim", int, at + ".mixer"))
+            if kind == "attention":
+                temp = m.get("q_temp")
+                coef, every = 0.0, 1
+                if temp is not None:
+                    coef = _require(temp, "coef", float, at + ".mixer.q_temp")
+                    every = temp.get("every")
+                    if isinstance(every, bool) or not isinstance(every, (int, float)) or every != int(every) or every <= 0:
+                        raise ConfigError(f"{at}.mixer.q_temp: 'every' must be a positive whole number, got {every!r}")
+                layers.append(NozuraxLayer(**common, kv_heads=_require(m, "kv_heads", int, at + ".mixer"),
+                                           scale=_require(m, "scale", float, at + ".mixer"), temp_coef=coef,
+                                           temp_every=int(every)))
+            elif kind == "retention":
+                decay = m.get("decay")
+                if not isinstance(decay, (list, tuple)) or any(isinstance(x, bool) or not isinstance(x, (int, float)) for x in decay):
+                    raise ConfigError(f"{at}.mixer: 'decay' must be a list of numbers, one per head")
+                rot = m.get("rot")
+                dims, base = 0, 10000.0
+                if rot is not None:
+                    dims = _require(rot, "dims", int, at + ".mixer.rot")
+                    base = _require(rot, "base", float, at + ".mixer.rot")
+                layers.append(NozuraxLayer(**common, decay=tuple(float(x) for x in decay), rot_dims=dims, rot_base=base))
+            else:
+                raise ConfigError(f"{at}: type must be 'attention' or 'retention', got {kind!r}")
+        norm = _section(d, "norm", where)
+        eos = d.get("eos_token_id")
+        eos = (eos,) if isinstance(eos, int) else tuple(int(x) for x in eos) if isinstance(eos, (list, tuple)) else None
+        cfg = cls(vocab=_require(d, "vocab", int, where), width=_require(d, "width", int, where),
+                  eps=_require(norm, "eps", float, where + ": norm"), layers=tuple(layers),
+                  dtype=canonical_dtype(d.get("dtype") or d.get("torch_dtype") or "bfloat16"), eos_token_id=eos,
+                  architecture=d.get("architecture") or (d.get("architectures") or ["Nozurax"])[0])
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab <= 0 or self.width <= 0:
+            raise ConfigError(f"config.json: vocab and width must be positive, got {self.vocab} and {self.width}")
+        if not (self.eps > 0):
+            raise ConfigError(f"config.json: norm.eps must be positive, got {self.eps}")
+        for i, layer in enumerate(self.layers):
+            at = f"config.json: layers[{i}]"
+            if min(layer.heads, layer.dim, layer.vdim) <= 0 or (layer.ff is not None and layer.ff <= 0):
+                raise ConfigError(f"{at}: heads, dim, vdim and ff must be positive")
+            j = layer.weights_of
+            if j != i:
+                if not 0 <= j < len(self.layers) or self.layers[j].weights_of != j:
+                    raise ConfigError(f"{at}: weights_of names layer {j}, which must exist and have tensors of its own")
+                own = self.layers[j]
+                if (own.kind, own.heads, own.dim, own.vdim, own.kv_heads, own.ff) != \
+                        (layer.kind, layer.heads, layer.dim, layer.vdim, layer.kv_heads, layer.ff):
+                    raise ConfigError(f"{at}: its sizes differ from those of layer {j}, whose tensors it runs")
+            if layer.kind == "attention":
+                if layer.kv_heads <= 0 or layer.heads % layer.kv_heads:
+                    raise ConfigError(f"{at}: {layer.heads} heads do not divide into {layer.kv_heads} kv_heads")
+            else:
+                if len(layer.decay) != layer.heads:
+                    raise ConfigError(f"{at}: {len(layer.decay)} decays for {layer.heads} heads")
+                if any(not 0.0 <= x <= 1.0 for x in layer.decay):
+                    raise ConfigError(f"{at}: a decay must lie in [0, 1]")
+                if layer.rot_dims % 2 or not 0 <= layer.rot_dims <= layer.dim or (layer.rot_dims and not layer.rot_base > 0):
+                    raise ConfigError(f"{at}: rot.dims {layer.rot_dims} must be even and at most dim {layer.dim}, rot.base positive")
+
+    def to_dict(self) -> dict:
+        """The config.json that describes this configuration."""
+        entries = []
+        for i, layer in enumerate(self.layers):
+            if layer.kind == "attention":
+                mixer = {"heads": layer.heads, "kv_heads": layer.kv_heads, "dim": layer.dim, "vdim": layer.vdim,
+                         "scale": layer.scale}
+                if layer.temp_coef:
+                    mixer["q_temp"] = {"coef": layer.temp_coef, "every": layer.temp_every}
+            else:
+                mixer = {"heads": layer.heads, "dim": layer.dim, "vdim": layer.vdim, "decay": list(layer.decay)}
+                if layer.rot_dims:
+                    mixer["rot"] = {"dims": layer.rot_dims, "base": layer.rot_base}
+            entry = {"type": layer.kind, "mixer": mixer,
+                     "mlp": None if layer.ff is None else {"kind": "dense", "ff": layer.ff}}
+            if layer.weights_of != i:
+                entry["weights_of"] = layer.weights_of
+            entries.append(entry)
+        out = {"architecture": self.architecture, "vocab": self.vocab, "width": self.width, "norm": {"eps": self.eps},
+               "layers": entries, "torch_dtype": self.dtype}
+        if self.eos_token_id is not None:
+            out["eos_token_id"] = list(self.eos_token_id)
+        return out

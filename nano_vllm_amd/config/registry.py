@@ -46,8 +46,10 @@ def get_architecture(name: str) -> Architecture:
 
 def architecture_of(config_json: Mapping[str, Any]) -> Architecture:
     names = config_json.get("architectures")
+    if not names and isinstance(config_json.get("architecture"), str):
+        names = [config_json["architecture"]]           # a config that names its one architecture as a string
     if not names or not isinstance(names, (list, tuple)):
-        raise ConfigError("config.json: key 'architectures' is missing or empty; "
+        raise ConfigError("config.json: key 'architectures' (or 'architecture') is missing or empty; "
                           f"known architectures: {known_architectures()}")
     return get_architecture(names[0])
 

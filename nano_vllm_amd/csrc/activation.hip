@@ -1,10 +1,22 @@
-// SwiGLU gating: out[t, i] = silu(x[t, i]) * x[t, inner + i], silu(g) = g * sigmoid(g)
-// (nanovllm/layers/activation.py:8-11).  Computed in float and rounded once.
+// Gating of a feed-forward: out[t, i] = act(x[t, i]) * x[t, inner + i].  SwiGLU is act = silu,
+// silu(g) = g * sigmoid(g) (nanovllm/layers/activation.py:8-11); the other activations are relu and
+// the tanh form of gelu, 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))).  Computed in float and
+// rounded once.
 #include "common.h"
 
-template <typename T, bool VEC>
+#define NVA_ACT_SILU 0
+#define NVA_ACT_RELU 1
+#define NVA_ACT_GELU_TANH 2
+
+template <int ACT> __device__ __forceinline__ float nva_act(float g) {
+    if (ACT == NVA_ACT_RELU) return fmaxf(g, 0.f);
+    if (ACT == NVA_ACT_GELU_TANH) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return g / (1.f + nva_exp(-g));
+}
+
+template <typename T, bool VEC, int ACT>
 __global__ void __launch_bounds__(256)
-silu_mul_kernel(const T* __restrict__ x, int64_t x_stride, T* __restrict__ out, int64_t out_stride, int inner) {
+act_mul_kernel(const T* __restrict__ x, int64_t x_stride, T* __restrict__ out, int64_t out_stride, int inner) {
     const int64_t row = blockIdx.y;
     const T* gate = x + row * x_stride;
     const T* up = gate + inner;
@@ -16,21 +28,22 @@ silu_mul_kernel(const T* __restrict__ x, int64_t x_stride, T* __restrict__ out, 
         load8(gate + i, g);
         load8(up + i, u);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) g[j] = g[j] / (1.f + nva_exp(-g[j])) * u[j];
+        for (int j = 0; j < 8; ++j) g[j] = nva_act<ACT>(g[j]) * u[j];
         store8(o + i, g);
     } else {
         const int i = blockIdx.x * blockDim.x + threadIdx.x;
         if (i >= inner) return;
         const float g = to_float(gate[i]);
-        o[i] = from_float<T>(g / (1.f + nva_exp(-g)) * to_float(up[i]));
+        o[i] = from_float<T>(nva_act<ACT>(g) * to_float(up[i]));
     }
 }
 
-NVA_EXPORT int NVA_NAME(nva_silu_mul)(const void* x, int64_t x_stride, void* out, int64_t out_stride,
-                                      int64_t rows, int inner, hipStream_t stream) {
+template <int ACT>
+static int launch_act_mul(const void* x, int64_t x_stride, void* out, int64_t out_stride, int64_t rows, int inner,
+                          hipStream_t stream) {
     if (rows == 0) return 0;
     if (rows < 0 || rows > 65535LL * 65535LL || inner <= 0)
-        return nva_fail("silu_mul: bad shape rows=%lld inner=%d", (long long)rows, inner);
+        return nva_fail("act_mul: bad shape rows=%lld inner=%d", (long long)rows, inner);
     const size_t vb = 8 * sizeof(elem_t);
     const bool vec = inner % 8 == 0 && x_stride % 8 == 0 && out_stride % 8 == 0 && nva_aligned(x, vb) &&
                      nva_aligned(out, vb);
@@ -41,15 +54,31 @@ NVA_EXPORT int NVA_NAME(nva_silu_mul)(const void* x, int64_t x_stride, void* out
         const unsigned nr = (unsigned)((rows - r0) < 65535 ? (rows - r0) : 65535);
         if (vec) {
             dim3 grid((inner / 8 + 255) / 256, nr);
-            hipLaunchKernelGGL((silu_mul_kernel<elem_t, true>), grid, dim3(256), 0, stream, xp + r0 * x_stride,
+            hipLaunchKernelGGL((act_mul_kernel<elem_t, true, ACT>), grid, dim3(256), 0, stream, xp + r0 * x_stride,
                                x_stride, op + r0 * out_stride, out_stride, inner);
         } else {
             dim3 grid((inner + 255) / 256, nr);
-            hipLaunchKernelGGL((silu_mul_kernel<elem_t, false>), grid, dim3(256), 0, stream, xp + r0 * x_stride,
+            hipLaunchKernelGGL((act_mul_kernel<elem_t, false, ACT>), grid, dim3(256), 0, stream, xp + r0 * x_stride,
                                x_stride, op + r0 * out_stride, out_stride, inner);
         }
     }
-    return nva_check_launch("silu_mul");
+    return nva_check_launch("act_mul");
+}
+
+// act: 0 silu, 1 relu, 2 gelu (tanh form)
+NVA_EXPORT int NVA_NAME(nva_act_mul)(const void* x, int64_t x_stride, void* out, int64_t out_stride,
+                                     int64_t rows, int inner, int act, hipStream_t stream) {
+    switch (act) {
+        case NVA_ACT_SILU: return launch_act_mul<NVA_ACT_SILU>(x, x_stride, out, out_stride, rows, inner, stream);
+        case NVA_ACT_RELU: return launch_act_mul<NVA_ACT_RELU>(x, x_stride, out, out_stride, rows, inner, stream);
+        case NVA_ACT_GELU_TANH: return launch_act_mul<NVA_ACT_GELU_TANH>(x, x_stride, out, out_stride, rows, inner, stream);
+    }
+    return nva_fail("act_mul: unknown activation %d", act);
+}
+
+NVA_EXPORT int NVA_NAME(nva_silu_mul)(const void* x, int64_t x_stride, void* out, int64_t out_stride,
+                                      int64_t rows, int inner, hipStream_t stream) {
+    return launch_act_mul<NVA_ACT_SILU>(x, x_stride, out, out_stride, rows, inner, stream);
 }
 
 NVA_DEFINE_LAST_ERROR(nva_activation)

@@ -11,6 +11,9 @@
 // s_j = scale * <q, k_j>, P = softmax(s), o = sum_j P_j v_j.  The step's own keys are in the
 // cache already when this runs.
 // Layouts: K [pages, Hkv, page, D], V transposed in tiles of keys (common.h).  One wave per (token, q head).
+// The values may have a size of their own, DV (V [pages, Hkv, page / vt, DV, vt], output rows of Hq * DV).
+// sinks, float [Hq] or null: a head's softmax has one more term exp(sink_h) in its denominator, a key
+// without a value that every query sees once; the running maximum starts at sink_h with a sum of 1.
 //
 // Portions of prompts have a second kernel with the same arithmetic, operation for operation (the
 // results are the same bits): a workgroup takes 32 query rows of one request and one head, and the
@@ -27,8 +30,8 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
                                const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                                const int32_t* __restrict__ block_tables, int table_stride,
                                const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
-                               int num_q_heads, int num_kv_heads, int head_dim, int page_size, float scale,
-                               int window, int32_t* error_flag) {
+                               int num_q_heads, int num_kv_heads, int head_dim, int v_dim, int page_size, float scale,
+                               int window, const float* __restrict__ sinks, int32_t* error_flag) {
     __shared__ float q_s[ATT_MAX_D];
     __shared__ float p_s[NVA_WAVE];
     __shared__ int64_t v_off_s[NVA_WAVE];
@@ -49,7 +52,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
     float acc[ATT_ACC];
 #pragma unroll
     for (int i = 0; i < ATT_ACC; ++i) acc[i] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
+    float m_run = sinks ? sinks[h] : -INFINITY, l_run = sinks ? 1.f : 0.f;
     const bool vec = head_dim % 8 == 0;
     const int vt = nva_v_tile(page_size);
 
@@ -65,7 +68,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
             } else {
                 const int64_t head_base = (int64_t)page * num_kv_heads + kvh;
                 const T* krow = k_cache + (head_base * page_size + off) * head_dim;
-                v_off = head_base * head_dim * (int64_t)page_size + nva_v_offset(off, 0, head_dim, vt);
+                v_off = head_base * v_dim * (int64_t)page_size + nva_v_offset(off, 0, v_dim, vt);
                 float dot = 0.f;
                 if (vec) {
                     int d = 0;
@@ -105,7 +108,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
 #pragma unroll
         for (int i = 0; i < ATT_ACC; ++i) {
             const int d = lane + i * NVA_WAVE;
-            if (d < head_dim) {
+            if (d < v_dim) {
                 float a = acc[i] * correction;
                 const T* vcol = v_cache + (int64_t)d * vt;
                 int jj = 0;
@@ -129,11 +132,11 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
         }
     }
     const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
-    T* orow = out + t * out_stride + (int64_t)h * head_dim;
+    T* orow = out + t * out_stride + (int64_t)h * v_dim;
 #pragma unroll
     for (int i = 0; i < ATT_ACC; ++i) {
         const int d = lane + i * NVA_WAVE;
-        if (d < head_dim) orow[d] = from_float<T>(acc[i] * inv);
+        if (d < v_dim) orow[d] = from_float<T>(acc[i] * inv);
     }
 }
 
@@ -145,8 +148,8 @@ template <int N> struct Count { static constexpr int value = N; };
 
 // floats of LDS the tiled kernel needs: the queries, a chunk of K (rows of an odd length: a lane per
 // key reads them side by side) and of V (channel-major, rows of 65)
-__host__ __device__ inline size_t att_tiled_lds(int head_dim) {
-    return ((size_t)ATT_ROWS * head_dim + (size_t)NVA_WAVE * (head_dim | 1) + (size_t)head_dim * (NVA_WAVE + 1)) * sizeof(float);
+__host__ __device__ inline size_t att_tiled_lds(int head_dim, int v_dim) {
+    return ((size_t)ATT_ROWS * head_dim + (size_t)NVA_WAVE * (head_dim | 1) + (size_t)v_dim * (NVA_WAVE + 1)) * sizeof(float);
 }
 
 template <typename T>
@@ -156,7 +159,8 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
                              const int32_t* __restrict__ block_tables, int table_stride,
                              const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ kv_lens,
                              const int32_t* __restrict__ tiles, int num_q_heads, int num_kv_heads, int head_dim,
-                             int page_size, float scale, int32_t* error_flag) {
+                             int v_dim, int page_size, float scale, const float* __restrict__ sinks,
+                             int32_t* error_flag) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     __shared__ int64_t k_off_s[NVA_WAVE], v_off_s[NVA_WAVE];       // of a chunk's keys; -1: the key has no page
     constexpr int ROWS_PER_WAVE = ATT_ROWS / ATT_TILED_WAVES;
@@ -164,7 +168,7 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
     const int DS = head_dim | 1;
     float* const q_s = lds;                                         // [ATT_ROWS][head_dim]
     float* const k_s = q_s + ATT_ROWS * head_dim;                   // [64 keys][DS]
-    float* const v_s = k_s + NVA_WAVE * DS;                         // [head_dim][65]
+    float* const v_s = k_s + NVA_WAVE * DS;                         // [v_dim][65]
 
     const int seq = tiles[2 * blockIdx.x], tile = tiles[2 * blockIdx.x + 1];
     const int h = blockIdx.y;
@@ -190,7 +194,7 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
     for (int r = 0; r < ROWS_PER_WAVE; ++r) {
 #pragma unroll
         for (int i = 0; i < ACC; ++i) acc[r][i] = 0.f;
-        m_run[r] = -INFINITY, l_run[r] = 0.f;
+        m_run[r] = sinks ? sinks[h] : -INFINITY, l_run[r] = sinks ? 1.f : 0.f;
     }
 
     for (int base = 0; base <= last_pos; base += NVA_WAVE) {
@@ -206,7 +210,7 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
                 } else {
                     const int64_t head_base = (int64_t)page * num_kv_heads + kvh;
                     k_off = (head_base * page_size + off) * head_dim;
-                    v_off = head_base * head_dim * (int64_t)page_size + nva_v_offset(off, 0, head_dim, vt);
+                    v_off = head_base * v_dim * (int64_t)page_size + nva_v_offset(off, 0, v_dim, vt);
                 }
             }
             k_off_s[tid] = k_off;
@@ -249,17 +253,17 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
             constexpr int B = 8;
             const int j = tid % NVA_WAVE;
             const int64_t v_off = v_off_s[j];
-            for (int d0 = tid / NVA_WAVE; d0 < head_dim; d0 += B * ATT_TILED_WAVES) {
+            for (int d0 = tid / NVA_WAVE; d0 < v_dim; d0 += B * ATT_TILED_WAVES) {
                 float vv[B];
 #pragma unroll
                 for (int u = 0; u < B; ++u) {
                     const int d = d0 + u * ATT_TILED_WAVES;
-                    vv[u] = d < head_dim && v_off >= 0 ? to_float(v_cache[v_off + (int64_t)d * vt]) : 0.f;
+                    vv[u] = d < v_dim && v_off >= 0 ? to_float(v_cache[v_off + (int64_t)d * vt]) : 0.f;
                 }
 #pragma unroll
                 for (int u = 0; u < B; ++u) {
                     const int d = d0 + u * ATT_TILED_WAVES;
-                    if (d < head_dim) v_s[d * (NVA_WAVE + 1) + j] = vv[u];
+                    if (d < v_dim) v_s[d * (NVA_WAVE + 1) + j] = vv[u];
                 }
             }
         }
@@ -334,7 +338,7 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
 #pragma unroll
                     for (int i = 0; i < ACC; ++i) {
                         const int dd = lane + i * NVA_WAVE;
-                        vv[i][u] = dd < head_dim ? v_s[dd * (NVA_WAVE + 1) + jj + u] : 0.f;
+                        vv[i][u] = dd < v_dim ? v_s[dd * (NVA_WAVE + 1) + jj + u] : 0.f;
                     }
                 }
 #pragma unroll
@@ -357,11 +361,11 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
         const int r = wave + ATT_TILED_WAVES * rr;
         if (r >= rows) continue;
         const float inv = l_run[rr] > 0.f ? 1.f / l_run[rr] : 0.f;
-        T* orow = out + (int64_t)(q_begin + q0 + r) * out_stride + (int64_t)h * head_dim;
+        T* orow = out + (int64_t)(q_begin + q0 + r) * out_stride + (int64_t)h * v_dim;
 #pragma unroll
         for (int i = 0; i < ACC; ++i) {
             const int d = lane + i * NVA_WAVE;
-            if (d < head_dim) orow[d] = from_float<T>(acc[rr][i] * inv);
+            if (d < v_dim) orow[d] = from_float<T>(acc[rr][i] * inv);
         }
     }
 }
@@ -372,51 +376,51 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
 NVA_EXPORT int NVA_NAME(nva_paged_attention_tiled)(
     const void* q, int64_t q_stride, void* out, int64_t out_stride, const void* k_cache, const void* v_cache,
     const int32_t* block_tables, int table_stride, const int32_t* cu_seqlens_q, const int32_t* kv_lens,
-    const int32_t* tiles, int64_t num_tiles, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
-    float scale, int32_t* error_flag, hipStream_t stream) {
+    const int32_t* tiles, int64_t num_tiles, int num_q_heads, int num_kv_heads, int head_dim, int v_dim,
+    int page_size, float scale, const float* sinks, int32_t* error_flag, hipStream_t stream) {
     if (num_tiles == 0) return 0;
-    if (head_dim <= 0 || head_dim > ATT_TILED_MAX_D) {
-        nva_fail("paged_attention_tiled: head_dim %d is outside 1..%d", head_dim, ATT_TILED_MAX_D);
+    if (head_dim <= 0 || head_dim > ATT_TILED_MAX_D || v_dim <= 0 || v_dim > ATT_TILED_MAX_D) {
+        nva_fail("paged_attention_tiled: head sizes %d / %d are outside 1..%d", head_dim, v_dim, ATT_TILED_MAX_D);
         return 1;
     }
     if (!tiles || num_tiles < 0 || num_tiles > 0x7fffffff) return nva_fail("paged_attention_tiled: bad tile count %lld", (long long)num_tiles);
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads || num_q_heads > 65535)
         return nva_fail("paged_attention_tiled: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
     if (page_size <= 0 || table_stride <= 0) return nva_fail("paged_attention_tiled: bad page size or table width");
-    const size_t lds = att_tiled_lds(head_dim);
+    const size_t lds = att_tiled_lds(head_dim, v_dim);
     auto kernel = paged_attention_tiled_kernel<elem_t>;
     static bool raised = false;              // the kernel's LDS limit, lifted once to what the largest head size needs
     if (!raised) {
-        if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)att_tiled_lds(ATT_TILED_MAX_D)) != hipSuccess)
-            return nva_fail("paged_attention_tiled: cannot have %zu bytes of LDS", att_tiled_lds(ATT_TILED_MAX_D));
+        if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)att_tiled_lds(ATT_TILED_MAX_D, ATT_TILED_MAX_D)) != hipSuccess)
+            return nva_fail("paged_attention_tiled: cannot have %zu bytes of LDS", att_tiled_lds(ATT_TILED_MAX_D, ATT_TILED_MAX_D));
         raised = true;
     }
     dim3 grid((unsigned)num_tiles, (unsigned)num_q_heads);
     hipLaunchKernelGGL(kernel, grid, dim3(ATT_TILED_WAVES * NVA_WAVE), lds, stream, (const elem_t*)q, q_stride,
                        (elem_t*)out, out_stride, (const elem_t*)k_cache, (const elem_t*)v_cache, block_tables,
-                       table_stride, cu_seqlens_q, kv_lens, tiles, num_q_heads, num_kv_heads, head_dim, page_size,
-                       scale, error_flag);
+                       table_stride, cu_seqlens_q, kv_lens, tiles, num_q_heads, num_kv_heads, head_dim, v_dim,
+                       page_size, scale, sinks, error_flag);
     return nva_check_launch("paged_attention_tiled");
 }
 
 NVA_EXPORT int NVA_NAME(nva_paged_attention_generic)(
     const void* q, int64_t q_stride, void* out, int64_t out_stride, const void* k_cache, const void* v_cache,
     const int32_t* block_tables, int table_stride, const int32_t* token_seq, const int32_t* positions,
-    int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, int page_size, float scale, int window,
-    int32_t* error_flag, hipStream_t stream) {
+    int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, int v_dim, int page_size, float scale,
+    int window, const float* sinks, int32_t* error_flag, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || tokens > 0x7fffffff) return nva_fail("paged_attention: bad token count %lld", (long long)tokens);
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads || num_q_heads > 65535)
         return nva_fail("paged_attention: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
-    if (head_dim <= 0 || head_dim > ATT_MAX_D)
-        return nva_fail("paged_attention: head_dim %d is outside 1..%d", head_dim, ATT_MAX_D);
+    if (head_dim <= 0 || head_dim > ATT_MAX_D || v_dim <= 0 || v_dim > ATT_MAX_D)
+        return nva_fail("paged_attention: head sizes %d / %d are outside 1..%d", head_dim, v_dim, ATT_MAX_D);
     if (page_size <= 0 || table_stride <= 0) return nva_fail("paged_attention: bad page size or table width");
     if (window < 0) return nva_fail("paged_attention: negative window");
     dim3 grid((unsigned)tokens, (unsigned)num_q_heads);
     hipLaunchKernelGGL(paged_attention_generic_kernel<elem_t>, grid, dim3(NVA_WAVE), 0, stream, (const elem_t*)q,
                        q_stride, (elem_t*)out, out_stride, (const elem_t*)k_cache, (const elem_t*)v_cache,
                        block_tables, table_stride, token_seq, positions, num_q_heads, num_kv_heads, head_dim,
-                       page_size, scale, window, error_flag);
+                       v_dim, page_size, scale, window, sinks, error_flag);
     return nva_check_launch("paged_attention_generic");
 }
 

@@ -173,4 +173,66 @@ NVA_EXPORT int NVA_NAME(nva_rms_norm_of_partials)(const float* sums, int splits,
     return launch<false>(nullptr, 0, part, nullptr, 0, weight, w_is_f32, (elem_t*)y, y_stride, rows, width, eps, stream);
 }
 
+// ---------------------------------------------------------------------------- float residual stream
+// The residual stream kept in float whatever the element type, with up to two addends a layer
+// (a block whose mixer and feed-forward read the same norm output and are added together):
+//     r <- a + b            (first: the stream starts here, r is not read)
+//     r <- r + a + b        (else; a and b may each be absent)
+//     y = r * rsqrt(mean(r^2) + eps) * (offset + w)        rounded once, to the element type
+// All arithmetic in float.  offset 1 is the weight stored around zero, offset 0 the plain weight.
+template <typename T>
+__global__ void __launch_bounds__(512)
+stream_rms_norm_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ b, int64_t b_stride,
+                       float* residual, int64_t r_stride, int first, const void* __restrict__ weight, int w_is_f32,
+                       float offset, T* __restrict__ y, int64_t y_stride, int width, float eps) {
+    __shared__ float scratch[16];
+    const int64_t row = blockIdx.x;
+    const T* ar = a ? a + row * a_stride : nullptr;
+    const T* br = b ? b + row * b_stride : nullptr;
+    float* rr = residual + row * r_stride;
+    T* yr = y + row * y_stride;
+    const T* w_e = static_cast<const T*>(weight);
+    const float* w_f = static_cast<const float*>(weight);
+    constexpr int KEEP = 4;                       // elements a thread keeps between the two passes
+    float kept[KEEP];
+    float ss = 0.f;
+    int n = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
+        float s = first ? 0.f : rr[i];
+        // the two sublayers are added to each other first, then to the stream
+        float add = 0.f;
+        if (ar) add = to_float(ar[i]);
+        if (br) add += to_float(br[i]);
+        s += add;
+        if (ar || br || first) rr[i] = s;
+        if (n < KEEP) kept[n] = s;
+        ss += s * s;
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = rsqrtf(ss / (float)width + eps);
+    n = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
+        const float s = n < KEEP ? kept[n] : rr[i];
+        const float w = offset + (w_is_f32 ? w_f[i] : to_float(w_e[i]));
+        yr[i] = from_float<T>(s * scale * w);
+    }
+}
+
+// residual: float [rows, width] in place.  a, b: elements or null.  first != 0: the stream starts with a (+ b).
+NVA_EXPORT int NVA_NAME(nva_stream_rms_norm)(const void* a, int64_t a_stride, const void* b, int64_t b_stride,
+                                             float* residual, int64_t r_stride, int first, const void* weight,
+                                             int w_is_f32, float offset, void* y, int64_t y_stride, int64_t rows,
+                                             int width, float eps, hipStream_t stream) {
+    if (rows == 0) return 0;
+    if (rows < 0 || rows > 0x7fffffff || width <= 0)
+        return nva_fail("stream_rms_norm: bad shape rows=%lld width=%d", (long long)rows, width);
+    if (!residual || !y || !weight) return nva_fail("stream_rms_norm: residual, output and weight are needed");
+    if (first && !a) return nva_fail("stream_rms_norm: the stream starts with an addend");
+    const int threads = width >= 2048 ? 512 : width >= 1024 ? 256 : width >= 256 ? 128 : 64;
+    hipLaunchKernelGGL((stream_rms_norm_kernel<elem_t>), dim3((unsigned)rows), dim3(threads), 0, stream,
+                       (const elem_t*)a, a_stride, (const elem_t*)b, b_stride, residual, r_stride, first, weight,
+                       w_is_f32, offset, (elem_t*)y, y_stride, width, eps);
+    return nva_check_launch("stream_rms_norm");
+}
+
 NVA_DEFINE_LAST_ERROR(nva_norm)

@@ -1,0 +1,204 @@
+// Retention: linear attention with a fixed decay per head, no softmax and no denominator.
+//
+// Per head, with a state S [D, DV] that starts at zero and is carried from token to token:
+//     q, k <- rotation of the first R channels in pairs (i, i + R/2) by the angle p * f_i
+//     k    <- k * k_scale
+//     S_t  = decay * S_(t-1) + k_t v_t^T          o_t = S_t^T q_t
+// and afterwards (the finishing kernel), per token and head,
+//     y = o / sqrt(mean(o^2) + eps) * silu(g)
+//
+// A step brings, for every request, one token or a portion of a prompt.  The portion is taken in
+// chunks of RET_C tokens.  With S the state before a chunk of n tokens and i, j its tokens:
+//     o_i  = decay^(i+1) S^T q_i + sum_{j <= i} decay^(i-j) (q_i . k_j) v_j
+//     S'   = decay^n S + sum_j decay^(n-1-j) k_j v_j^T
+// No quotient of powers is ever taken, so small decays do not overflow.  The columns of S (the value
+// channels) do not depend on each other: a workgroup takes one request, one head and a slice of
+// value channels, keeps its part of S in LDS over all the chunks, and writes it back at the end.
+//
+// Everything here is float: the rotation (angles from the float position and float frequencies,
+// accurate sine and cosine), the scores, the decay powers (a table [heads, RET_C + 1] made on the
+// host in double), the state and the sums.  Only the projections are read as elements, and the
+// finished y is rounded once.
+//
+// The step's metadata is read on the device only (cu_seqlens_q, seq_starts, state_slots), so a
+// captured step replays for other requests.  seq_starts[s] == 0 starts from a zero state.
+#include "common.h"
+
+#define RET_C 32                  // tokens of a chunk
+#define RET_THREADS 256
+#define RET_MAX_VSLICE 32         // value channels of a workgroup
+
+__host__ __device__ inline size_t ret_lds_floats(int dim, int vslice) {
+    // q and k [RET_C][dim + 1], v [RET_C][vslice], scores [RET_C][RET_C + 1], state [dim][vslice]
+    return (size_t)2 * RET_C * (dim + 1) + (size_t)RET_C * vslice + (size_t)RET_C * (RET_C + 1) + (size_t)dim * vslice;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(RET_THREADS)
+retention_chunk_kernel(const T* __restrict__ proj, int64_t stride, float* __restrict__ o_raw, int64_t o_stride,
+                       float* __restrict__ state, const int32_t* __restrict__ cu_seqlens_q,
+                       const int32_t* __restrict__ seq_starts, const int32_t* __restrict__ state_slots,
+                       const float* __restrict__ decay_pow, const float* __restrict__ inv_freq, int rot,
+                       int heads, int dim, int vdim, int vslice, int nslices, float k_scale) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int DS = dim + 1;
+    float* const q_s = lds;                              // [RET_C][DS]
+    float* const k_s = q_s + RET_C * DS;                 // [RET_C][DS]
+    float* const v_s = k_s + RET_C * DS;                 // [RET_C][vslice]
+    float* const a_s = v_s + RET_C * vslice;             // [RET_C][RET_C + 1]
+    float* const s_s = a_s + RET_C * (RET_C + 1);        // [dim][vslice]
+
+    const int h = blockIdx.x / nslices, slice = blockIdx.x % nslices;
+    const int seq = blockIdx.y;
+    const int c0 = slice * vslice;
+    const int nc = min(vslice, vdim - c0);               // this slice's channels
+    const int tid = threadIdx.x;
+    const int q_begin = cu_seqlens_q[seq];
+    const int q_len = cu_seqlens_q[seq + 1] - q_begin;
+    const int start = seq_starts[seq];
+    const int slot = state_slots[seq];
+    const float* pw = decay_pow + (int64_t)h * (RET_C + 1);
+    float* const s_g = state + (((int64_t)slot * heads + h) * dim) * vdim + c0;      // [dim][vdim] of (slot, head), at this slice
+    const int half = rot / 2;
+    const int64_t q_off = (int64_t)h * dim, k_off = (int64_t)(heads + h) * dim;
+    const int64_t v_off = (int64_t)2 * heads * dim + (int64_t)h * vdim + c0;
+
+    for (int e = tid; e < dim * nc; e += RET_THREADS) {
+        const int d = e / nc, c = e % nc;
+        s_s[d * vslice + c] = start > 0 ? s_g[(int64_t)d * vdim + c] : 0.f;
+    }
+
+    for (int t0 = 0; t0 < q_len; t0 += RET_C) {
+        const int n = min(RET_C, q_len - t0);
+        __syncthreads();                                 // the chunk before is done with q, k, v and the scores
+        // ---- q and k of the chunk, rotated, k scaled; v
+        for (int e = tid; e < n * dim; e += RET_THREADS) {
+            const int r = e / dim, d = e % dim;
+            const T* row = proj + (int64_t)(q_begin + t0 + r) * stride;
+            float qv = to_float(row[q_off + d]), kv = to_float(row[k_off + d]);
+            if (d < rot) {
+                const bool lower = d < half;
+                const int partner = lower ? d + half : d - half;
+                const float angle = (float)(start + t0 + r) * inv_freq[lower ? d : d - half];
+                float sn, cs;
+                sincosf(angle, &sn, &cs);
+                const float qp = to_float(row[q_off + partner]), kp = to_float(row[k_off + partner]);
+                qv = lower ? qv * cs - qp * sn : qv * cs + qp * sn;
+                kv = lower ? kv * cs - kp * sn : kv * cs + kp * sn;
+            }
+            q_s[r * DS + d] = qv;
+            k_s[r * DS + d] = kv * k_scale;
+        }
+        for (int e = tid; e < n * nc; e += RET_THREADS) {
+            const int r = e / nc, c = e % nc;
+            v_s[r * vslice + c] = to_float(proj[(int64_t)(q_begin + t0 + r) * stride + v_off + c]);
+        }
+        __syncthreads();
+        // ---- scores of the chunk with their decay: a[i][j] = decay^(i-j) q_i . k_j for j <= i
+        for (int e = tid; e < n * n; e += RET_THREADS) {
+            const int i = e / n, j = e % n;
+            float dot = 0.f;
+            if (j <= i) {
+                const float* qi = q_s + i * DS;
+                const float* kj = k_s + j * DS;
+                for (int d = 0; d < dim; ++d) dot += qi[d] * kj[d];
+                dot *= pw[i - j];
+            }
+            a_s[i * (RET_C + 1) + j] = dot;
+        }
+        __syncthreads();
+        // ---- outputs: what the state before the chunk gives, and the chunk's own tokens
+        for (int e = tid; e < n * nc; e += RET_THREADS) {
+            const int i = e / nc, c = e % nc;
+            const float* qi = q_s + i * DS;
+            float from_state = 0.f;
+            for (int d = 0; d < dim; ++d) from_state += qi[d] * s_s[d * vslice + c];
+            float own = 0.f;
+            const float* ai = a_s + i * (RET_C + 1);
+            for (int j = 0; j <= i; ++j) own += ai[j] * v_s[j * vslice + c];
+            o_raw[(int64_t)(q_begin + t0 + i) * o_stride + (int64_t)h * vdim + c0 + c] = pw[i + 1] * from_state + own;
+        }
+        __syncthreads();
+        // ---- the state after the chunk
+        const float all = pw[n];
+        for (int e = tid; e < dim * nc; e += RET_THREADS) {
+            const int d = e / nc, c = e % nc;
+            float add = 0.f;
+            for (int j = 0; j < n; ++j) add += pw[n - 1 - j] * k_s[j * DS + d] * v_s[j * vslice + c];
+            s_s[d * vslice + c] = all * s_s[d * vslice + c] + add;
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < dim * nc; e += RET_THREADS) {
+        const int d = e / nc, c = e % nc;
+        s_g[(int64_t)d * vdim + c] = s_s[d * vslice + c];
+    }
+}
+
+// y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * silu(g[t, h, :]); one wave per (token, head).
+template <typename T>
+__global__ void __launch_bounds__(NVA_WAVE)
+retention_finish_kernel(const float* __restrict__ o_raw, int64_t o_stride, const T* __restrict__ gate, int64_t g_stride,
+                        T* __restrict__ y, int64_t y_stride, int vdim, float eps) {
+    const int64_t t = blockIdx.x;
+    const int h = blockIdx.y, lane = threadIdx.x;
+    const float* o = o_raw + t * o_stride + (int64_t)h * vdim;
+    const T* g = gate + t * g_stride + (int64_t)h * vdim;
+    T* out = y + t * y_stride + (int64_t)h * vdim;
+    float ss = 0.f;
+    for (int c = lane; c < vdim; c += NVA_WAVE) ss += o[c] * o[c];
+    ss = wave_sum(ss);
+    const float scale = rsqrtf(ss / (float)vdim + eps);
+    for (int c = lane; c < vdim; c += NVA_WAVE) {
+        const float gv = to_float(g[c]);
+        out[c] = from_float<T>(o[c] * scale * (gv / (1.f + expf(-gv))));
+    }
+}
+
+// proj: [tokens, 2 * heads * dim + 2 * heads * vdim] = [q | k | v | g], rows `stride` elements apart.
+// o_raw: float [tokens, heads * vdim] scratch.  y: [tokens, heads * vdim] elements.
+// state: float [slots, heads, dim, vdim].  decay_pow: float [heads, RET_C + 1], decay_h^m.
+// inv_freq: float [rot / 2] (rot 0: no rotation).  vslice: value channels per workgroup (1..32).
+NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* o_raw, void* y, int64_t y_stride,
+                                       float* state, int64_t num_slots, const int32_t* cu_seqlens_q,
+                                       const int32_t* seq_starts, const int32_t* state_slots, int64_t num_seqs,
+                                       int64_t tokens, const float* decay_pow, const float* inv_freq, int rot,
+                                       int heads, int dim, int vdim, int vslice, float k_scale, float eps,
+                                       hipStream_t stream) {
+    if (num_seqs == 0 || tokens == 0) return 0;
+    if (num_seqs < 0 || num_seqs > 65535 || tokens < 0 || tokens > 0x7fffffff)
+        return nva_fail("retention: bad counts requests=%lld tokens=%lld", (long long)num_seqs, (long long)tokens);
+    if (heads <= 0 || heads > 65535 || dim <= 0 || vdim <= 0 || vslice <= 0 || vslice > RET_MAX_VSLICE)
+        return nva_fail("retention: bad sizes heads=%d dim=%d vdim=%d vslice=%d", heads, dim, vdim, vslice);
+    if (rot < 0 || rot % 2 || rot > dim || (rot && !inv_freq))
+        return nva_fail("retention: %d rotated channels of a head of %d", rot, dim);
+    const int64_t width = (int64_t)2 * heads * dim + (int64_t)2 * heads * vdim;
+    if (stride < width || y_stride < (int64_t)heads * vdim) return nva_fail("retention: rows are too short");
+    if (!proj || !o_raw || !y || !state || !cu_seqlens_q || !seq_starts || !state_slots || !decay_pow || num_slots <= 0)
+        return nva_fail("retention: a needed tensor is missing");
+    const int nslices = (vdim + vslice - 1) / vslice;
+    if ((int64_t)heads * nslices > 0x7fffffff) return nva_fail("retention: too many workgroups");
+    const size_t lds = ret_lds_floats(dim, vslice) * sizeof(float);
+    if (lds > 160 * 1024) return nva_fail("retention: a head of %d channels does not fit the LDS", dim);
+    auto kernel = retention_chunk_kernel<elem_t>;
+    static size_t raised = 48 * 1024;
+    if (lds > raised) {
+        if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+            return nva_fail("retention: cannot have %zu bytes of LDS", lds);
+        raised = 160 * 1024;
+    }
+    const elem_t* p = (const elem_t*)proj;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(heads * nslices), (unsigned)num_seqs), dim3(RET_THREADS), lds, stream, p,
+                       stride, o_raw, (int64_t)heads * vdim, state, cu_seqlens_q, seq_starts, state_slots, decay_pow,
+                       inv_freq, rot, heads, dim, vdim, vslice, nslices, k_scale);
+    int rc = nva_check_launch("retention");
+    if (rc) return rc;
+    const elem_t* gate = p + (int64_t)2 * heads * dim + (int64_t)heads * vdim;
+    hipLaunchKernelGGL((retention_finish_kernel<elem_t>), dim3((unsigned)tokens, (unsigned)heads), dim3(NVA_WAVE), 0, stream,
+                       o_raw, (int64_t)heads * vdim, gate, stride, (elem_t*)y, y_stride, vdim, eps);
+    return nva_check_launch("retention_finish");
+}
+
+NVA_EXPORT int NVA_NAME(nva_retention_chunk)() { return RET_C; }
+
+NVA_DEFINE_LAST_ERROR(nva_retention)

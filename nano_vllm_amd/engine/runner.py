@@ -222,7 +222,9 @@ def load_model(folder: str, dtype: Optional[str] = None, device="cuda:0", kernel
     spec = arch.build_spec(config)
     tdtype = torch_dtype(dtype or spec.dtype)
     if kernels is None:
-        kernels = HipKernels(device, tdtype, quiet=quiet)        # raises without a GPU or the compiled kernels
+        # only what this model's parts call is compiled now (raises without a GPU or a compiler)
+        modules = Model(spec, None, "cpu", tdtype).kernel_modules()
+        kernels = HipKernels(device, tdtype, quiet=quiet, modules=modules)
     model = Model(spec, kernels, device, tdtype)
     if random_weights is None:
         load_weights(model, folder)

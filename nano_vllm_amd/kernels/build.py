@@ -36,6 +36,8 @@ MODULES: Dict[str, Tuple[str, Tuple[Optional[str], ...]]] = {
     "attn_decode": ("attn_decode.hip", ("bf16",)),
     "attn_prefill": ("attn_prefill.hip", ("bf16",)),
     "sample": ("sample.hip", (None,)),
+    "qk_rownorm": ("qk_rownorm.hip", ("bf16", "f32")),
+    "retention": ("retention.hip", ("bf16", "f32")),
 }
 
 _HEADERS = ("common.h",)
@@ -187,10 +189,13 @@ def all_targets() -> List[Tuple[str, Optional[str]]]:
     return [(m, d) for m, (_, dtypes) in MODULES.items() for d in dtypes]
 
 
-def targets_for(dtype: str) -> List[Tuple[str, Optional[str]]]:
-    """What a model of one element type ("bf16" or "f32") needs."""
+def targets_for(dtype: str, modules: Optional[Iterable[str]] = None) -> List[Tuple[str, Optional[str]]]:
+    """What a model of one element type ("bf16" or "f32") needs: every module built for that type,
+    or those of `modules` that are."""
     out = []
     for m, (_, dtypes) in MODULES.items():
+        if modules is not None and m not in modules:
+            continue
         if dtype in dtypes:
             out.append((m, dtype))
         elif None in dtypes:

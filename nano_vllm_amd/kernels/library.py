@@ -23,6 +23,7 @@ _LAST_ERROR_SYMBOL = {
     "sample": "nva_sample_last_error", "attn_decode": "nva_attn_decode_last_error",
     "gemm_skinny": "nva_gemm_skinny_last_error", "gemm_team": "nva_gemm_team_last_error",
     "attn_prefill": "nva_attn_prefill_last_error", "gemm_tile": "nva_gemm_tile_last_error",
+    "qk_rownorm": "nva_qk_rownorm_last_error", "retention": "nva_retention_last_error",
 }
 
 _loaded: Dict[Tuple[str, Optional[str]], ctypes.CDLL] = {}
@@ -42,9 +43,10 @@ def load(module: str, dtype: Optional[str]) -> ctypes.CDLL:
     return lib
 
 
-def preload(dtype: str, quiet: bool = False) -> None:
-    """Builds (in parallel) and loads everything a model of this element type calls."""
-    targets = build.targets_for(dtype)
+def preload(dtype: str, quiet: bool = False, modules=None) -> None:
+    """Builds (in parallel) and loads everything a model of this element type calls: every module,
+    or the named ones (a model's parts say which they call; anything else is built when first called)."""
+    targets = build.targets_for(dtype, modules)
     build.ensure_built(targets, quiet=quiet)
     for m, d in targets:
         load(m, d)

@@ -205,7 +205,9 @@ class HipKernels:
     name = "hip"
     max_burst_groups = 4        # cache groups nva_advance_decode takes in one launch
 
-    def __init__(self, device="cuda:0", dtype: torch.dtype = torch.bfloat16, quiet: bool = False):
+    def __init__(self, device="cuda:0", dtype: torch.dtype = torch.bfloat16, quiet: bool = False, modules=None):
+        """modules: the kernel modules to compile and load now (None: all of the element type);
+        whatever else is called later is compiled then."""
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: the engine runs on HIP kernels only and has no CPU path")
         if dtype not in _SUFFIX:
@@ -213,7 +215,7 @@ class HipKernels:
         self.device = torch.device(device)
         self.dtype = dtype
         self.suffix = _SUFFIX[dtype]
-        library.preload(self.suffix, quiet=quiet)       # compiles what this element type needs
+        library.preload(self.suffix, quiet=quiet, modules=modules)       # compiles what this element type needs
         # bit 0: a token id outside the vocabulary; bit 1: a visible key without a page;
         # bit 2: the decode attention's plan outgrew its bound
         self.fault_flag = torch.zeros(1, dtype=torch.int32, device=self.device)
@@ -357,21 +359,80 @@ class HipKernels:
                      c_i32(wf), _p(out), c_i64(os_), c_i64(rows), c_i32(width), c_f32(eps), self._stream())
         return out, residual
 
+    def stream_rms_norm(self, addends, residual: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                        offset: float = 0.0, out: Optional[torch.Tensor] = None):
+        """The norm of a residual stream that is kept in float32 whatever the element type:
+        residual <- residual + sum(addends) in place (residual None: a new stream that starts as the
+        sum of the addends), then y = residual * rsqrt(mean(residual^2) + eps) * (offset + weight),
+        all in float and rounded once.  addends: up to two tensors of the element type [rows, width].
+        Returns (y, residual)."""
+        addends = [_t(a) for a in addends]
+        if len(addends) > 2 or (residual is None and not addends):
+            raise KernelError("stream_rms_norm: one or two addends (none only with a stream that exists)")
+        ref = addends[0] if addends else None
+        if ref is None:
+            if out is None:
+                raise KernelError("stream_rms_norm: without addends the output tensor says the element type")
+            rows, width = residual.shape
+        else:
+            rows, width, _ = _rows2d(ref, "stream_rms_norm addend")
+        strides = []
+        for a in addends:
+            ar, aw, as_ = _rows2d(a, "stream_rms_norm addend")
+            if (ar, aw) != (rows, width) or a.dtype != ref.dtype:
+                raise KernelError("stream_rms_norm: the addends differ in shape or type")
+            strides.append(as_)
+        first = residual is None
+        if first:
+            residual = torch.empty((rows, width), dtype=torch.float32, device=ref.device)
+        rrows, rw, rs = _rows2d(residual, "stream_rms_norm residual")
+        if (rrows, rw) != (rows, width) or residual.dtype != torch.float32:
+            raise KernelError("stream_rms_norm: the residual stream must be float32 of the addends' shape")
+        dtype = ref.dtype if ref is not None else out.dtype
+        if out is None:
+            out = torch.empty((rows, width), dtype=dtype, device=residual.device)
+        orows, ow, os_ = _rows2d(out, "stream_rms_norm output")
+        if (orows, ow) != (rows, width) or out.dtype != dtype:
+            raise KernelError("stream_rms_norm: output does not match")
+        wf = self._norm_weight(weight, width, out)
+        a = addends[0] if addends else None
+        b = addends[1] if len(addends) > 1 else None
+        library.call("norm", _suffix(out), "nva_stream_rms_norm", _p(a), c_i64(strides[0] if addends else 0), _p(b),
+                     c_i64(strides[1] if len(addends) > 1 else 0), _p(residual), c_i64(rs), c_i32(1 if first else 0),
+                     _p(weight), c_i32(wf), c_f32(offset), _p(out), c_i64(os_), c_i64(rows), c_i32(width), c_f32(eps),
+                     self._stream())
+        return out, residual
+
     # ------------------------------------------------------------------ feed-forward
-    def silu_mul(self, gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+
+    def act_mul(self, gate_up: torch.Tensor, act: str = "silu", out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """act(gate) * up of a row [gate | up]; act: silu, relu or gelu_tanh."""
+        if act not in self.ACTIVATIONS:
+            raise KernelError(f"act_mul: unknown activation {act!r}; known: {sorted(self.ACTIVATIONS)}")
         gate_up = _t(gate_up)
-        rows, width, xs = _rows2d(gate_up, "silu_mul input")
+        rows, width, xs = _rows2d(gate_up, "act_mul input")
         if width % 2:
-            raise KernelError("silu_mul: the input holds gate and up halves, its width must be even")
+            raise KernelError("act_mul: the input holds gate and up halves, its width must be even")
         inner = width // 2
         if out is None:
             out = torch.empty((rows, inner), dtype=gate_up.dtype, device=gate_up.device)
-        orows, ow, os_ = _rows2d(out, "silu_mul output")
+        orows, ow, os_ = _rows2d(out, "act_mul output")
         if (orows, ow) != (rows, inner) or out.dtype != gate_up.dtype:
-            raise KernelError("silu_mul: output does not match the input")
-        library.call("activation", _suffix(gate_up), "nva_silu_mul", _p(gate_up), c_i64(xs), _p(out), c_i64(os_),
-                     c_i64(rows), c_i32(inner), self._stream())
+            raise KernelError("act_mul: output does not match the input")
+        library.call("activation", _suffix(gate_up), "nva_act_mul", _p(gate_up), c_i64(xs), _p(out), c_i64(os_),
+                     c_i64(rows), c_i32(inner), c_i32(self.ACTIVATIONS[act]), self._stream())
         return out
+
+    def silu_mul(self, gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return self.act_mul(gate_up, "silu", out=out)
+
+    def linear_act_mul(self, x: torch.Tensor, weight: torch.Tensor, act: str = "silu") -> torch.Tensor:
+        """act(x @ Wg.T) * (x @ Wu.T) with weight = [Wg; Wu].  silu has the gating in the products'
+        epilogues (linear_silu_mul); the other activations run the product and the gating kernel."""
+        if act == "silu":
+            return self.linear_silu_mul(x, weight)
+        return self.act_mul(self.linear(x, weight), act)
 
     # ------------------------------------------------------------------ matrix products
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -816,13 +877,50 @@ class HipKernels:
                      _p(k_cache), _p(v_cache), c_i32(page_size), self._stream())
         return q
 
+    def qk_rownorm_store(self, qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int,
+                         q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                         positions: Optional[torch.Tensor], temp_coef: float, temp_every: int,
+                         slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                         v_cache: Optional[torch.Tensor]) -> torch.Tensor:
+        """q and k normed over the whole projection (all heads at once, plain weights [heads * head_dim]
+        and [kv_heads * head_dim]), q scaled by the temperature 1 + temp_coef * ln(floor((p + 1) /
+        temp_every) + 1) of its position p, both written back in place, k and v written into their page
+        slots.  The row is [q | k | v] with values of v_head_dim.  Returns the q view."""
+        qkv = _t(qkv)
+        tokens, width, stride = _rows2d(qkv, "qkv")
+        want = (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_head_dim
+        if width != want:
+            raise KernelError(f"qkv width {width} is not heads * head_dim + kv_heads * (head_dim + v_head_dim) = {want}")
+        wf = 0
+        for w, n in ((q_weight, num_heads * head_dim), (k_weight, num_kv_heads * head_dim)):
+            if w is not None:
+                wf = self._norm_weight(w, n, qkv)
+        if num_kv_heads and (q_weight is None) != (k_weight is None):
+            raise KernelError("qk norm: give both weights or none")
+        if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
+            raise KernelError("qk norm: the two weights differ in type")
+        if temp_coef:
+            if positions is None or int(temp_every) <= 0:
+                raise KernelError("a query temperature needs the positions and a positive step")
+            _i32(positions, tokens, "positions")
+        page_size = 0
+        if k_cache is not None:
+            page_size = self._check_cache(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype, v_head_dim)
+            _i32(slots, tokens, "slots")
+        library.call("qk_rownorm", _suffix(qkv), "nva_qk_rownorm_store", _p(qkv), c_i64(stride), c_i64(tokens),
+                     c_i32(num_heads), c_i32(num_kv_heads), c_i32(head_dim), c_i32(v_head_dim), _p(q_weight), _p(k_weight),
+                     c_i32(wf), c_f32(eps), _p(positions), c_f32(float(temp_coef)), c_i32(int(temp_every) if temp_coef else 1),
+                     _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size), self._stream())
+        return qkv[:, : num_heads * head_dim]
+
     @staticmethod
-    def _check_cache(k_cache, v_cache, num_kv_heads, head_dim, dtype) -> int:
+    def _check_cache(k_cache, v_cache, num_kv_heads, head_dim, dtype, v_head_dim=None) -> int:
         if k_cache.dim() != 4 or v_cache is None or v_cache.dim() != 5:
             raise KernelError("cache tensors must be K [pages, kv_heads, page, head_dim] and "
-                              "V [pages, kv_heads, page / vt, head_dim, vt]")
+                              "V [pages, kv_heads, page / vt, v_head_dim, vt]")
         pages, h, page_size, d = k_cache.shape
-        if (h, d) != (num_kv_heads, head_dim) or tuple(v_cache.shape) != v_cache_shape(pages, h, d, page_size):
+        vd = head_dim if v_head_dim is None else v_head_dim
+        if (h, d) != (num_kv_heads, head_dim) or tuple(v_cache.shape) != v_cache_shape(pages, h, vd, page_size):
             raise KernelError(f"cache shapes K {tuple(k_cache.shape)} V {tuple(v_cache.shape)} do not fit "
                               f"{num_kv_heads} kv heads of {head_dim}")
         if not (k_cache.is_contiguous() and v_cache.is_contiguous()) or k_cache.dtype != dtype or v_cache.dtype != dtype:
@@ -832,14 +930,21 @@ class HipKernels:
     # ------------------------------------------------------------------ attention
     def paged_attention(self, q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                         k_cache: torch.Tensor, v_cache: torch.Tensor, batch, group: int, scale: float,
-                        window: Optional[int] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                        window: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                        v_head_dim: Optional[int] = None, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Causal attention of the step's tokens over the cache.  `batch` is the step's
-        StepBatch; `group` selects its block tables.  q [T, heads*head_dim] (rows may be strided)."""
+        StepBatch; `group` selects its block tables.  q [T, heads*head_dim] (rows may be strided).
+        v_head_dim: the size of a head's values where it is not head_dim (the output is then
+        [T, heads*v_head_dim]).  sinks, float32 [heads]: one more term exp(sink_h) in the denominator
+        of head h's softmax, a key without a value that every query sees once."""
         q = _t(q)
         tokens, width, qs = _rows2d(q, "attention q")
         if width != num_heads * head_dim:
             raise KernelError("attention: q width is not heads * head_dim")
-        page_size = self._check_cache(k_cache, v_cache, num_kv_heads, head_dim, q.dtype)
+        v_dim = head_dim if v_head_dim is None else int(v_head_dim)
+        if sinks is not None and (sinks.dtype != torch.float32 or sinks.shape != (num_heads,) or not sinks.is_contiguous()):
+            raise KernelError(f"attention: sinks must be contiguous float32 [{num_heads}]")
+        page_size = self._check_cache(k_cache, v_cache, num_kv_heads, head_dim, q.dtype, v_dim)
         if num_heads % num_kv_heads:
             raise KernelError(f"attention: {num_heads} heads do not divide into {num_kv_heads} kv heads")
         tables = batch.groups[group].block_tables
@@ -851,9 +956,9 @@ class HipKernels:
         if tables.shape[1] < need_pages:
             raise KernelError(f"attention: block tables hold {tables.shape[1]} pages, {need_pages} are needed")
         if out is None:
-            out = torch.empty((tokens, width), dtype=q.dtype, device=q.device)
+            out = torch.empty((tokens, num_heads * v_dim), dtype=q.dtype, device=q.device)
         _, ow, os_ = _rows2d(out, "attention out")
-        if ow != width or out.shape[0] != tokens or out.dtype != q.dtype:
+        if ow != num_heads * v_dim or out.shape[0] != tokens or out.dtype != q.dtype:
             raise KernelError("attention: output does not match q")
         if any(n != 1 for n in batch.q_lens[:batch.num_decode]):
             raise KernelError("attention: the first num_decode requests of a batch must bring one token each")
@@ -861,7 +966,8 @@ class HipKernels:
         # them where its shape limits allow; everything else runs the general kernel
         start = 0
         # (the matrix-core kernels fold the scale into the exponent, which needs it positive)
-        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf")
+        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and \
+            v_dim == head_dim and sinks is None
         if batch.num_decode > 0 and mfma and \
                 self._decode_kernel_takes(num_heads // num_kv_heads, head_dim, page_size, q, qs, out, os_):
             start = batch.num_decode
@@ -878,22 +984,76 @@ class HipKernels:
                          _p(self.fault_flag), self._stream())
             start = tokens
         if self.tiled_general_attention and start <= batch.num_decode < tokens and not window and \
-                head_dim <= GENERAL_TILED_MAX_HEAD_DIM:
+                max(head_dim, v_dim) <= GENERAL_TILED_MAX_HEAD_DIM:
             # portions of prompts in float arithmetic: the per-token kernel's arithmetic, operation for
             # operation, with the keys staged once for 32 query rows
             tiles = self._prefill_tiles(batch, q.device)
             library.call("attn_generic", _suffix(q), "nva_paged_attention_tiled", _p(q), c_i64(qs), _p(out), c_i64(os_),
                          _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.cu_seqlens_q),
                          _p(batch.kv_lens), _p(tiles), c_i64(tiles.shape[0]), c_i32(num_heads), c_i32(num_kv_heads),
-                         c_i32(head_dim), c_i32(page_size), c_f32(scale), _p(self.fault_flag), self._stream())
+                         c_i32(head_dim), c_i32(v_dim), c_i32(page_size), c_f32(scale), _p(sinks), _p(self.fault_flag),
+                         self._stream())
             tokens = batch.num_decode            # what is left: the single tokens before the portions
         if start < tokens:
             n = tokens - start
             library.call("attn_generic", _suffix(q), "nva_paged_attention_generic", _p(q[start:start + n]), c_i64(qs),
                          _p(out[start:]), c_i64(os_), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
                          _p(batch.token_seq[start:]), _p(batch.positions[start:]), c_i64(n), c_i32(num_heads),
-                         c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
-                         _p(self.fault_flag), self._stream())
+                         c_i32(num_kv_heads), c_i32(head_dim), c_i32(v_dim), c_i32(page_size), c_f32(scale),
+                         c_i32(window or 0), _p(sinks), _p(self.fault_flag), self._stream())
+        return out
+
+    # ------------------------------------------------------------------ retention
+    RETENTION_CHUNK = 32        # tokens of a chunk of nva_retention (the rows of its table of decay powers, less one)
+
+    def retention(self, proj: torch.Tensor, heads: int, dim: int, v_dim: int, state: torch.Tensor,
+                  decay_powers: torch.Tensor, inv_freq: Optional[torch.Tensor], k_scale: float, eps: float,
+                  batch, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Retention of the step's tokens: proj [T, 2*heads*dim + 2*heads*v_dim] = [q | k | v | g];
+        per head S <- decay S + k v^T, o = S^T q with q and k rotated by their position (inv_freq
+        float32 [rot/2], None: no rotation) and k scaled by k_scale; then o / rms(o) * silu(g) per
+        head.  state: float32 [slots, heads, dim, v_dim], a request's row given by batch.state_slots,
+        started from zero where batch.seq_starts is 0.  decay_powers: float32 [heads, RETENTION_CHUNK + 1],
+        decay_h^m.  Returns [T, heads*v_dim] of proj's type."""
+        proj = _t(proj)
+        tokens, width, stride = _rows2d(proj, "retention projections")
+        if width != 2 * heads * (dim + v_dim):
+            raise KernelError(f"retention: projections of width {width}, expected 2 * heads * (dim + v_dim) = "
+                              f"{2 * heads * (dim + v_dim)}")
+        if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, v_dim) or \
+                not state.is_contiguous():
+            raise KernelError(f"retention: the state must be contiguous float32 [slots, {heads}, {dim}, {v_dim}]")
+        if decay_powers.dtype != torch.float32 or tuple(decay_powers.shape) != (heads, self.RETENTION_CHUNK + 1) or \
+                not decay_powers.is_contiguous():
+            raise KernelError(f"retention: decay powers must be contiguous float32 [{heads}, {self.RETENTION_CHUNK + 1}]")
+        rot = 0
+        if inv_freq is not None:
+            if inv_freq.dtype != torch.float32 or inv_freq.dim() != 1 or not inv_freq.is_contiguous():
+                raise KernelError("retention: inv_freq must be contiguous float32")
+            rot = 2 * inv_freq.shape[0]
+            if rot > dim:
+                raise KernelError(f"retention: {rot} rotated channels of a head of {dim}")
+        seqs = batch.num_seqs
+        _i32(batch.cu_seqlens_q, seqs + 1, "cu_seqlens_q")
+        _i32(batch.seq_starts, seqs, "seq_starts")
+        _i32(batch.state_slots, seqs, "state_slots")
+        if sum(batch.q_lens) != tokens:
+            raise KernelError("retention: the batch does not describe the projections' rows")
+        if out is None:
+            out = torch.empty((tokens, heads * v_dim), dtype=proj.dtype, device=proj.device)
+        orows, ow, os_ = _rows2d(out, "retention output")
+        if (orows, ow) != (tokens, heads * v_dim) or out.dtype != proj.dtype:
+            raise KernelError("retention: output does not match")
+        raw = torch.empty((tokens, heads * v_dim), dtype=torch.float32, device=proj.device)
+        # value channels per workgroup: fewer where that is needed to give every CU a workgroup
+        vslice = 32
+        while vslice > 8 and seqs * heads * ((v_dim + vslice - 1) // vslice) < self.cus:
+            vslice //= 2
+        vslice = min(vslice, max(1, v_dim))
+        library.call("retention", _suffix(proj), "nva_retention", _p(proj), c_i64(stride), _p(raw), _p(out), c_i64(os_),
+                     _p(state), c_i64(state.shape[0]), _p(batch.cu_seqlens_q), _p(batch.seq_starts),
+                     _p(batch.state_slots), c_i64(seqs), c_i64(tokens), _p(decay_powers), _p(inv_freq), c_i32(rot),
+                     c_i32(heads), c_i32(dim), c_i32(v_dim), c_i32(vslice), c_f32(k_scale), c_f32(eps), self._stream())
         return out
 
     @staticmethod

@@ -1,1 +1,2 @@
 from . import qwen3  # noqa: F401  (registers Qwen3ForCausalLM)
+from . import nozurax  # noqa: F401  (registers Nozurax)

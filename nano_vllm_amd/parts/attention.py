@@ -8,6 +8,13 @@
     cache <- k, v                   (attention.py:62-63)
     o = softmax(scale q K^T) V      causal, over the request's cached keys, optionally a window
     out = o Wo^T                    (qwen3.py:87)
+Options beyond the reference's attention, each a parameter:
+    v_head_dim                      values of a size of their own (the output heads have that size)
+    qk_norm_scope "projection"      q and k normed over the whole projection, all heads at once, with
+                                    weights of that size, before the split into heads
+    q_temperature (coef, every)     q *= 1 + coef * ln(floor((p + 1) / every) + 1) at position p
+    sink                            a learned number per head whose exponential joins the softmax's
+                                    denominator: a key without a value that every query sees once
 
 Interface of a mixer:
     cache_need()                 -> PagedKV | FixedState | None
@@ -27,7 +34,9 @@ class Attention(Part):
     """params: hidden_size, num_heads, num_kv_heads, head_dim, qk_norm (bool), eps, bias (bool),
     position_encoding (a name in the model's position encodings, or None), window (None or
     keys), scale (None: head_dim^-0.5), reads_shared_cache (bool: the run owns no cache, it
-    projects q only and reads another run's keys and values)."""
+    projects q only and reads another run's keys and values), v_head_dim (None: head_dim),
+    qk_norm_scope ("head" | "projection"), q_temperature (None or {"coef", "every"}), sink (bool),
+    and the names of the checkpoint tensors (q_name, ..., q_norm_name, k_norm_name, sink_name)."""
 
     def __init__(self, params: Mapping, build: BuildContext):
         super().__init__(params, build)
@@ -50,31 +59,65 @@ class Attention(Part):
         self.q_name, self.k_name, self.v_name = (p.get("q_name", "q_proj"), p.get("k_name", "k_proj"),
                                                  p.get("v_name", "v_proj"))
         self.o_name = p.get("o_name", "o_proj")
+        self.q_norm_name, self.k_norm_name = p.get("q_norm_name", "q_norm"), p.get("k_norm_name", "k_norm")
+        self.sink_name = p.get("sink_name", "sinks")
+        v = p.get("v_head_dim")
+        self.v_head_dim = self.head_dim if v is None else int(v)
+        self.norm_scope = p.get("qk_norm_scope", "head")
+        if self.norm_scope not in ("head", "projection"):
+            raise ValueError(f"attention: qk_norm_scope must be 'head' or 'projection', got {self.norm_scope!r}")
+        temp = p.get("q_temperature")
+        self.temp_coef = float(temp["coef"]) if temp else 0.0
+        self.temp_every = int(temp["every"]) if temp else 1
+        self.sink = bool(p.get("sink", False))
+        # The whole-projection preparation has its own kernel, which also scales q by its temperature
+        # and stores values of their own size; the per-head one rotates.  Each does what its model needs.
+        self.row_prepare = self.norm_scope == "projection" or self.temp_coef != 0.0 or self.v_head_dim != self.head_dim
+        if self.row_prepare and self.position_encoding is not None:
+            raise ValueError("attention: a position encoding goes with per-head norms, equal head sizes and no "
+                             "query temperature")
+        if self.row_prepare and self.qk_norm and self.norm_scope == "head":
+            raise ValueError("attention: per-head norms go with equal head sizes and no query temperature")
+
+    @property
+    def kernel_modules(self):
+        prepare = "qk_rownorm" if self.row_prepare else "rope"
+        if self.sink or self.v_head_dim != self.head_dim:
+            return (prepare, "attn_generic")
+        return (prepare, "attn_generic", "attn_decode", "attn_prefill")
 
     # ------------------------------------------------------------------ declaration
     def param_decls(self) -> Dict[str, ParamDecl]:
         q, kv, h = self.heads * self.head_dim, self.kv_heads * self.head_dim, self.hidden
+        vv = self.kv_heads * self.v_head_dim
         d: Dict[str, ParamDecl] = {}
         if self.shared:
             shards = ((self.q_name, 0, q),)
             rows = q
         else:
-            shards = ((self.q_name, 0, q), (self.k_name, q, kv), (self.v_name, q + kv, kv))
-            rows = q + 2 * kv
+            shards = ((self.q_name, 0, q), (self.k_name, q, kv), (self.v_name, q + kv, vv))
+            rows = q + kv + vv
         d["qkv_proj.weight"] = ParamDecl((rows, h), sources=tuple(Source(f"{n}.weight", r, c) for n, r, c in shards))
         if self.bias:
             d["qkv_proj.bias"] = ParamDecl((rows,), sources=tuple(Source(f"{n}.bias", r, c) for n, r, c in shards))
         if self.qk_norm:
-            d["q_norm.weight"] = ParamDecl((self.head_dim,), dtype="stored32", init="norm")
+            whole = self.norm_scope == "projection"
+            qn, kn = (q, kv) if whole else (self.head_dim, self.head_dim)
+            d["q_norm.weight"] = ParamDecl((qn,), dtype="stored32", init="norm",
+                                           sources=(Source(f"{self.q_norm_name}.weight", 0, qn),))
             if not self.shared:
-                d["k_norm.weight"] = ParamDecl((self.head_dim,), dtype="stored32", init="norm")
-        d[f"{self.o_name}.weight"] = ParamDecl((h, q))
+                d["k_norm.weight"] = ParamDecl((kn,), dtype="stored32", init="norm",
+                                               sources=(Source(f"{self.k_norm_name}.weight", 0, kn),))
+        if self.sink:
+            d["sinks"] = ParamDecl((self.heads,), dtype="float32", sources=(Source(self.sink_name, 0, self.heads),))
+        d[f"{self.o_name}.weight"] = ParamDecl((h, self.heads * self.v_head_dim))
         return d
 
     def cache_need(self):
         if self.shared:
             return None
-        return PagedKV(self.kv_heads, self.head_dim, self.window)
+        return PagedKV(self.kv_heads, self.head_dim, self.window,
+                       None if self.v_head_dim == self.head_dim else self.v_head_dim)
 
     # ------------------------------------------------------------------ forward
     def forward(self, x, batch, cache):
@@ -84,13 +127,17 @@ class Attention(Part):
         # deferred: the products below are handed to the q/k preparation and to the block's norm only
         pe = self.position_encoding
         table = pe.rotary_table() if pe is not None else None
-        qkv = k.linear(x, w["qkv_proj.weight"], w.get("qkv_proj.bias"), deferred=pe is None or table is not None)
+        qkv = k.linear(x, w["qkv_proj.weight"], w.get("qkv_proj.bias"),
+                       deferred=not self.row_prepare and (pe is None or table is not None))
         group = batch.groups[cache.group]
         slots = None if self.shared else group.slot_mapping
         kc, vc = (None, None) if self.shared else (cache.k, cache.v)
         qw = w.get("q_norm.weight")
         kw = w.get("k_norm.weight")
-        if pe is None or table is not None:
+        if self.row_prepare:
+            q = k.qk_rownorm_store(qkv, self.heads, kv_heads, self.head_dim, self.v_head_dim, qw, kw, self.eps,
+                                   batch.positions, self.temp_coef, self.temp_every, slots, kc, vc)
+        elif pe is None or table is not None:
             q = k.qk_norm_rope_store(qkv, self.heads, kv_heads, self.head_dim, qw, kw, self.eps, table,
                                      batch.positions, slots, kc, vc, max_position=batch.max_kv_len)
         else:
@@ -103,8 +150,12 @@ class Attention(Part):
             if not self.shared:
                 k.qk_norm_rope_store(qkv, self.heads, kv_heads, self.head_dim, None, None, self.eps, None, None,
                                      slots, kc, vc)
-        o = k.paged_attention(q, self.heads, self.kv_heads, self.head_dim, cache.k, cache.v, batch, cache.group,
-                              self.scale, self.window)
+        if self.sink or self.v_head_dim != self.head_dim:
+            o = k.paged_attention(q, self.heads, self.kv_heads, self.head_dim, cache.k, cache.v, batch, cache.group,
+                                  self.scale, self.window, v_head_dim=self.v_head_dim, sinks=w.get("sinks"))
+        else:
+            o = k.paged_attention(q, self.heads, self.kv_heads, self.head_dim, cache.k, cache.v, batch, cache.group,
+                                  self.scale, self.window)
         return k.linear(o, w[f"{self.o_name}.weight"], deferred=True)
 
 

@@ -50,6 +50,11 @@ class Part:
     # state slot of their own that no request holds (the state tensors' last row).
     replays_state_steps = False
 
+    # The kernel modules (kernels.build.MODULES) this part calls beyond those every model calls
+    # (rows, norms, products, gating): they are compiled together before the model's first step.
+    # What a part calls without naming it here is compiled when first called.
+    kernel_modules: Tuple[str, ...] = ()
+
     def __init__(self, params: Mapping, build: BuildContext):
         self.params = dict(params)
         self.kernels = build.kernels

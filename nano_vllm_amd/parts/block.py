@@ -7,7 +7,15 @@ next norm (nanovllm/models/qwen3.py:146-159):
     a = mixer(x);  r = a + r;  y = norm2(r);  m = feed_forward(y);  returns (m, r)
 The caller adds the last m to r inside the final norm (qwen3.py:182).
 
-Interface of a block: forward(h, residual | None, batch, cache) -> (h, residual).
+"parallel_residual": one norm whose output both sublayers read, their sum added to the stream:
+    x = norm(r);  r <- r + (mixer(x) + feed_forward(x))
+The residual stream r is float32 whatever the element type.  The sum is deferred into the next
+norm as well: the block returns the two sublayer outputs as a list of addends with the stream as
+it was before them, and the next block's norm (or the model's final norm) adds them.  The first
+block gets the embedding as its one addend.  A layer may have no feed-forward.
+
+Interface of a block: forward(h, residual | None, batch, cache) -> (h, residual); h is a tensor,
+or a list of addends for a float32 stream.
 """
 from __future__ import annotations
 
@@ -54,4 +62,39 @@ class PreNormResidualBlock(Part):
         return m, residual
 
 
+class ParallelResidualBlock(Part):
+    ROLES = ("norm", "mixer", "feed_forward")
+
+    def __init__(self, params: Mapping, build: BuildContext):
+        super().__init__(params, build)
+        parts = params["parts"]
+        names = params["names"]
+        missing = [r for r in ("norm", "mixer") if r not in parts]
+        if missing:
+            raise ValueError(f"parallel_residual block: missing parts {missing}")
+        self.norm = make_part("norm", parts["norm"], build)
+        self.mixer = make_part("mixer", parts["mixer"], build)
+        self.feed_forward = make_part("feed_forward", parts["feed_forward"], build) if parts.get("feed_forward") else None
+        self._children = {names[r]: getattr(self, r) for r in self.ROLES if getattr(self, r) is not None}
+
+    def children(self) -> Dict[str, Part]:
+        return self._children
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def replays_state_steps(self):
+        return self.mixer.replays_state_steps
+
+    def forward(self, h, residual, batch, cache):
+        addends = h if isinstance(h, (tuple, list)) else (h,)
+        x, residual = self.norm.forward_add(addends, residual)
+        a = self.mixer.forward(x, batch, cache)
+        if self.feed_forward is None:
+            return (a,), residual
+        return (a, self.feed_forward.forward(x, batch)), residual
+
+
 register_part("block", "pre_norm_residual", PreNormResidualBlock)
+register_part("block", "parallel_residual", ParallelResidualBlock)

@@ -91,6 +91,22 @@ class Model:
         for part in [*self.position_encodings.values(), self.embedding, *self.blocks, self.final_norm, self.head]:
             told(part)
 
+    BASE_KERNEL_MODULES = ("embed", "norm", "activation", "gemm", "gemm_skinny", "gemm_team", "gemm_tile")
+
+    def kernel_modules(self):
+        """The kernel modules this model's steps call: what every model calls and what its parts name."""
+        found = list(self.BASE_KERNEL_MODULES)
+
+        def walk(part: Part) -> None:
+            for m in part.kernel_modules:
+                if m not in found:
+                    found.append(m)
+            for child in part.children().values():
+                walk(child)
+        for part in [*self.position_encodings.values(), self.embedding, *self.blocks, self.final_norm, self.head]:
+            walk(part)
+        return tuple(found)
+
     def num_parameters(self) -> int:
         return sum(int(torch.tensor(d.shape).prod()) for _, _, d in self.param_table.values())
 

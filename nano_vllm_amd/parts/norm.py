@@ -2,6 +2,11 @@
 
 "rms_norm": y = cast(x * rsqrt(mean(x^2) + eps)) * weight, and the same fused with the
 residual sum (nanovllm/layers/layernorm.py:16-40).  Sizes and eps are parameters.
+
+With weight_offset c the factor is (c + weight): c = 1 is the weight stored around zero.  A norm
+with an offset, and every norm that is handed a list of addends instead of one tensor, works on a
+residual stream kept in float32: the stream takes the sum of the addends, the norm is computed in
+float and rounded once to the element type.
 """
 from __future__ import annotations
 
@@ -12,22 +17,31 @@ from .registry import register_part
 
 
 class RMSNorm(Part):
-    """params: dim, eps."""
+    """params: dim, eps, weight_offset (default 0)."""
 
     def __init__(self, params: Mapping, build: BuildContext):
         super().__init__(params, build)
         self.dim = int(params["dim"])
         self.eps = float(params["eps"])
+        self.offset = float(params.get("weight_offset", 0.0))
 
     def param_decls(self) -> Dict[str, ParamDecl]:
         # vectors stay in float32 when the checkpoint stores them so
-        return {"weight": ParamDecl((self.dim,), dtype="stored32", init="norm")}
+        # (a weight that is stored around zero is drawn around zero in random-weights mode)
+        return {"weight": ParamDecl((self.dim,), dtype="stored32", init="norm" if self.offset == 0.0 else "normal")}
 
     def forward(self, x, out=None):
+        if self.offset != 0.0:
+            return self.kernels.stream_rms_norm((x,), None, self.weights["weight"], self.eps, self.offset, out=out)[0]
         return self.kernels.rms_norm(x, self.weights["weight"], self.eps, out=out)
 
     def forward_add(self, x, residual, out=None):
-        """residual <- x + residual; returns (norm(residual), residual)."""
+        """residual <- x + residual; returns (norm(residual), residual).  x may be a list of one or
+        two addends: the residual is then a float32 stream (None: it starts as their sum)."""
+        if isinstance(x, (tuple, list)):
+            return self.kernels.stream_rms_norm(tuple(x), residual, self.weights["weight"], self.eps, self.offset, out=out)
+        if self.offset != 0.0:
+            raise ValueError("rms_norm: a weight offset goes with a float32 residual stream (a list of addends)")
         return self.kernels.add_rms_norm(x, residual, self.weights["weight"], self.eps, out=out)
 
 

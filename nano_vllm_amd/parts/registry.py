@@ -35,4 +35,4 @@ def known_parts(role: str):
 
 
 def _load_builtin() -> None:
-    from . import norm, rotary, attention, feed_forward, block, embedding  # noqa: F401
+    from . import norm, rotary, attention, retention, feed_forward, block, embedding  # noqa: F401

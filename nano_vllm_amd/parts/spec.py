@@ -66,6 +66,16 @@ class ModelSpec:
     head: PartSpec                               # params: name, tied
     position_encodings: Mapping[str, PartSpec]   # shared by name among the mixers
     eos_token_ids: Tuple[int, ...] = ()
+    # How the checkpoint names its tensors where that is not "<part>.<parameter>": pairs (suffix,
+    # replacement) tried in turn on every derived name, the first that fits is applied
+    # ((".weight", "") for a checkpoint that calls a matrix by its part's name alone).
+    checkpoint_names: Tuple[Tuple[str, str], ...] = ()
+
+    def checkpoint_name(self, derived: str) -> str:
+        for suffix, replacement in self.checkpoint_names:
+            if derived.endswith(suffix):
+                return derived[: len(derived) - len(suffix)] + replacement
+        return derived
 
     def validate(self) -> None:
         for i, run in enumerate(self.order):
@@ -83,10 +93,15 @@ class ModelSpec:
 class PagedKV:
     """Keys and values of every token, in pages.  window None: all keys stay; an integer:
     a query at position p reads positions > p - window only, and pages wholly before that
-    are given back."""
+    are given back.  v_head_dim: the size of a head's values where it is not head_dim."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
 
 @dataclass(frozen=True)

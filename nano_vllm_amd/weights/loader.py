@@ -52,13 +52,16 @@ class Slot:
 def checkpoint_layout(model) -> Dict[str, Slot]:
     """checkpoint tensor name -> Slot, from the parameters the model's parts declare."""
     layout: Dict[str, Slot] = {}
+    called = getattr(model.spec, "checkpoint_name", lambda name: name)      # the checkpoint's own way of naming
     for full, (_, local, decl) in model.param_table.items():
         prefix = full[: len(full) - len(local)]          # ends with "."
         if decl.sources is None:
-            layout[full] = Slot(full, 0, decl.shape[0] if decl.shape else 1, tuple(decl.shape), True)
+            if called(full) in layout:
+                raise ValueError(f"two parameters claim the checkpoint tensor {called(full)!r}")
+            layout[called(full)] = Slot(full, 0, decl.shape[0] if decl.shape else 1, tuple(decl.shape), True)
         else:
             for src in decl.sources:
-                name = prefix + src.name
+                name = called(prefix + src.name)
                 if name in layout:
                     raise ValueError(f"two parameters claim the checkpoint tensor {name!r}")
                 layout[name] = Slot(full, src.row, src.rows, (src.rows,) + tuple(decl.shape[1:]), False)
@@ -82,7 +85,7 @@ def load_weights(model, folder: str) -> None:
     if not files:
         raise WeightError(other=[f"{folder!r} holds no *.safetensors file"])
     layout = checkpoint_layout(model)
-    tied_head = model.spec.head["name"] + ".weight" if getattr(model.head, "tied", False) else None
+    tied_head = model.spec.checkpoint_name(model.spec.head["name"] + ".weight") if getattr(model.head, "tied", False) else None
     seen, unexpected, wrong = set(), [], []
     tensors: Dict[str, torch.Tensor] = {}
     tied_copy = None

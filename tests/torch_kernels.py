@@ -19,11 +19,11 @@ def v_tile(page_size: int) -> int:
     return 32 if page_size % 32 == 0 else page_size
 
 
-def new_caches(pages, kv_heads, head_dim, page_size, dtype, device, fill=None):
-    """K [pages, kv_heads, page, head_dim] and V [pages, kv_heads, page / vt, head_dim, vt]."""
+def new_caches(pages, kv_heads, head_dim, page_size, dtype, device, fill=None, v_head_dim=None):
+    """K [pages, kv_heads, page, head_dim] and V [pages, kv_heads, page / vt, v_head_dim, vt]."""
     vt = v_tile(page_size)
     k = torch.zeros((pages, kv_heads, page_size, head_dim), dtype=dtype, device=device)
-    v = torch.zeros((pages, kv_heads, page_size // vt, head_dim, vt), dtype=dtype, device=device)
+    v = torch.zeros((pages, kv_heads, page_size // vt, v_head_dim or head_dim, vt), dtype=dtype, device=device)
     if fill is not None:
         k.normal_(0, fill)
         v.normal_(0, fill)
@@ -71,15 +71,45 @@ class TorchKernels:
             return out, residual
         return y, residual
 
+    def stream_rms_norm(self, addends, residual, weight, eps, offset=0.0, out=None):
+        """The float32 residual stream takes the sum of the addends; its norm, in float, rounded once."""
+        add = None
+        for a in addends:
+            add = a.float() if add is None else add + a.float()
+        if residual is None:
+            residual = add.clone()
+        elif add is not None:
+            residual += add
+        dt = addends[0].dtype if addends else out.dtype
+        y = (residual * torch.rsqrt(residual.pow(2).mean(-1, keepdim=True) + eps) * (offset + weight.float())).to(dt)
+        if out is not None:
+            out.copy_(y)
+            return out, residual
+        return y, residual
+
     # feed-forward (activation.py:8-11)
-    def silu_mul(self, gate_up, out=None):
+    def act_mul(self, gate_up, act="silu", out=None):
         inner = gate_up.shape[1] // 2
         g, u = gate_up[:, :inner].float(), gate_up[:, inner:].float()
-        y = (g * torch.sigmoid(g) * u).to(gate_up.dtype)
+        if act == "silu":
+            a = g * torch.sigmoid(g)
+        elif act == "relu":
+            a = torch.relu(g)
+        elif act == "gelu_tanh":
+            a = 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))
+        else:
+            raise ValueError(act)
+        y = (a * u).to(gate_up.dtype)
         if out is not None:
             out.copy_(y)
             return out
         return y
+
+    def silu_mul(self, gate_up, out=None):
+        return self.act_mul(gate_up, "silu", out)
+
+    def linear_act_mul(self, x, weight, act="silu"):
+        return self.act_mul(self.linear(x, weight), act)
 
     def linear(self, x, weight, bias=None, out_float32=False, out=None, deferred=False):
         y = x.float() @ weight.float().T
@@ -138,14 +168,80 @@ class TorchKernels:
                 v_cache[page, :, off // vt, :, off % vt] = v[ok]
         return qkv[:, :qd]
 
+    def qk_rownorm_store(self, qkv, num_heads, num_kv_heads, head_dim, v_head_dim, q_weight, k_weight, eps,
+                         positions, temp_coef, temp_every, slots, k_cache, v_cache):
+        """q and k normed over the whole projection, q times its position's temperature, k and v stored."""
+        T = qkv.shape[0]
+        qd, kd = num_heads * head_dim, num_kv_heads * head_dim
+        dt = qkv.dtype
+        q = qkv[:, :qd].float()
+        if q_weight is not None:
+            q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_weight.float()
+        if temp_coef:
+            steps = torch.div(positions.long() + 1, int(temp_every), rounding_mode="floor").float()
+            q = q * (1.0 + temp_coef * torch.log(steps + 1.0))[:, None]
+        qkv[:, :qd] = q.to(dt)
+        if num_kv_heads:
+            k = qkv[:, qd:qd + kd].float()
+            if k_weight is not None:
+                k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_weight.float()
+            qkv[:, qd:qd + kd] = k.to(dt)
+            if k_cache is not None:
+                page_size, vt = k_cache.shape[2], v_cache.shape[4]
+                s = slots.long()
+                ok = s >= 0
+                page, off = s[ok] // page_size, s[ok] % page_size
+                k_cache[page, :, off, :] = qkv[:, qd:qd + kd].reshape(T, num_kv_heads, head_dim)[ok]
+                v_cache[page, :, off // vt, :, off % vt] = qkv[:, qd + kd:].reshape(T, num_kv_heads, v_head_dim)[ok]
+        return qkv[:, :qd]
+
+    RETENTION_CHUNK = 4
+
+    def retention(self, proj, heads, dim, v_dim, state, decay_powers, inv_freq, k_scale, eps, batch, out=None):
+        """Token by token: S <- decay S + k v^T, o = S^T q, then o / rms(o) * silu(g) per head."""
+        T = proj.shape[0]
+        qk, vv = heads * dim, heads * v_dim
+        p = proj.float()
+        q, k = p[:, :qk].reshape(T, heads, dim), p[:, qk:2 * qk].reshape(T, heads, dim)
+        v, g = p[:, 2 * qk:2 * qk + vv].reshape(T, heads, v_dim), p[:, 2 * qk + vv:]
+        pos = torch.cat([torch.arange(s, s + n) for s, n in zip(batch.starts, batch.q_lens)]).to(proj.device)
+        if inv_freq is not None:
+            half = inv_freq.shape[0]
+            ang = pos.float()[:, None] * inv_freq[None, :]
+            cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+
+            def turn(x):
+                a, b = x[..., :half], x[..., half:2 * half]
+                return torch.cat((a * cos - b * sin, b * cos + a * sin, x[..., 2 * half:]), dim=-1)
+            q, k = turn(q), turn(k)
+        k = k * k_scale
+        decay = decay_powers[:, 1].float()
+        o = torch.zeros((T, heads, v_dim), dtype=torch.float32, device=proj.device)
+        t = 0
+        slots = batch.state_slots.tolist()
+        for s, (start, n) in enumerate(zip(batch.starts, batch.q_lens)):
+            S = state[slots[s]].clone() if start > 0 else torch.zeros_like(state[slots[s]])
+            for i in range(t, t + n):
+                S = decay[:, None, None] * S + k[i][:, :, None] * v[i][:, None, :]
+                o[i] = torch.einsum("hdv,hd->hv", S, q[i])
+            state[slots[s]] = S
+            t += n
+        o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+        y = (o.reshape(T, vv) * (g * torch.sigmoid(g))).to(proj.dtype)
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
+
     # attention (attention.py:64-75): token by token through the block table
     def paged_attention(self, q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, batch, group, scale,
-                        window=None, out=None):
+                        window=None, out=None, v_head_dim=None, sinks=None):
         T = q.shape[0]
         D, G = head_dim, num_heads // num_kv_heads
+        DV = v_head_dim or head_dim
         page_size = k_cache.shape[2]
         tables = batch.groups[group].block_tables
-        o = torch.zeros((T, num_heads * D), dtype=torch.float32, device=q.device)
+        o = torch.zeros((T, num_heads * DV), dtype=torch.float32, device=q.device)
         pos_l, seq_l = batch.positions.tolist(), batch.token_seq.tolist()
         for t in range(T):
             pos, seq = pos_l[t], seq_l[t]
@@ -160,8 +256,11 @@ class TorchKernels:
             qt = q[t].float().reshape(num_heads, D)
             for h in range(num_heads):
                 s = (keys[:, h // G] @ qt[h]) * scale
-                p = torch.softmax(s, dim=0)
-                o[t, h * D:(h + 1) * D] = p @ vals[:, h // G]
+                if sinks is not None:       # one more term in the denominator: a key without a value
+                    p = torch.softmax(torch.cat((s, sinks[h:h + 1].float())), dim=0)[:-1]
+                else:
+                    p = torch.softmax(s, dim=0)
+                o[t, h * DV:(h + 1) * DV] = p @ vals[:, h // G]
         y = o.to(q.dtype)
         if out is not None:
             out.copy_(y)
