@@ -17,6 +17,13 @@ temperature 0.6, ignore_eos, one `generate` call after a short warm-up request) 
 
 One JSON line is printed: `value` is decoded tokens a second at the default batch.
 The reference measures throughput the same way on synthetic token ids (bench.py:8-28 there).
+
+    python bench.py --design nozurax [--design-sizes 1024,2048,4096] [--layers 4]
+
+is another measurement and leaves the default one as it is: prefill and decode throughput of the
+Nozurax design (alternating attention and retention layers) beside a Qwen3 model of the same layer
+sizes, a few layers of each with random weights, through the same step function; one JSON line
+with both designs' numbers per size.
 """
 import argparse
 import json
@@ -48,7 +55,118 @@ def parse_args():
                     help="context of one more decode point at the default batch (0: none)")
     ap.add_argument("--serve-seqs", type=int, default=256,
                     help="requests of the reference's benchmark workload through LLM.generate (0: not run)")
+    ap.add_argument("--design", default=None, choices=["nozurax"],
+                    help="measure this design beside Qwen3 at equal layer sizes instead of the default workload")
+    ap.add_argument("--design-sizes", default="1024,2048,4096", help="model widths of the --design measurement")
     return ap.parse_args()
+
+
+# layer sizes of the --design measurement by width: (query heads, kv heads, head size, inner size): those of
+# the Qwen3 0.6B, 1.7B and 8B shapes
+DESIGN_SIZES = {1024: (16, 8, 128, 3072), 2048: (16, 8, 128, 6144), 4096: (32, 8, 128, 12288)}
+DESIGN_VOCAB = 32768
+
+
+def design_configs(width: int, layers: int, dtype: str):
+    """config.json of a Nozurax model and of the Qwen3 model with the same layer sizes."""
+    heads, kv, dim, inner = DESIGN_SIZES[width]
+    att = {"type": "attention", "mlp": {"kind": "dense", "ff": inner},
+           "mixer": {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                     "q_temp": {"coef": 0.1, "every": 256}}}
+    ret = {"type": "retention", "mlp": {"kind": "dense", "ff": inner},
+           "mixer": {"heads": heads, "dim": dim, "vdim": dim, "rot": {"dims": dim, "base": 1e6},
+                     "decay": [1.0 - 2.0 ** (-5 - 3.0 * h / heads) for h in range(heads)]}}
+    nozurax = {"architecture": "Nozurax", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6},
+               "layers": [att if i % 2 == 0 else ret for i in range(layers)], "torch_dtype": dtype}
+    qwen3 = {"architectures": ["Qwen3ForCausalLM"], "hidden_size": width, "num_hidden_layers": layers,
+             "num_attention_heads": heads, "num_key_value_heads": kv, "head_dim": dim, "intermediate_size": inner,
+             "vocab_size": DESIGN_VOCAB, "rms_norm_eps": 1e-6, "rope_theta": 1e6, "max_position_embeddings": 40960,
+             "tie_word_embeddings": False, "attention_bias": False, "hidden_act": "silu", "torch_dtype": dtype}
+    return {"nozurax": nozurax, "qwen3": qwen3}
+
+
+def design_run(args):
+    """Prefill and decode throughput of the design and of Qwen3 at equal sizes, layer for layer."""
+    import torch
+    from nano_vllm_amd.config import architecture_of
+    from nano_vllm_amd.engine.batch import StepEntry
+    from nano_vllm_amd.engine.runner import ModelRunner
+    from nano_vllm_amd.kernels import HipKernels
+    from nano_vllm_amd.parts.model import Model, torch_dtype
+    from nano_vllm_amd.weights import fill_random_
+    device, dtype = "cuda:0", torch_dtype(args.dtype)
+    kernels = HipKernels(device, dtype)
+    layers = args.layers or 4
+    T, B, ctx, page = args.prefill_tokens, args.batch, args.context, args.page_size
+    gen = torch.Generator().manual_seed(args.seed)
+    out = {}
+    for width in [int(w) for w in args.design_sizes.split(",") if w]:
+        out[width] = {}
+        for name, config_json in design_configs(width, layers, args.dtype).items():
+            arch = architecture_of(config_json)
+            model = Model(arch.build_spec(arch.parse_config(config_json)), kernels, device, dtype)
+            fill_random_(model, args.seed)
+            pages = B * ((ctx + page - 1) // page + 1) + (T + page - 1) // page + 1
+            runner = ModelRunner(model, page, pages, B + 1, enable_prefix_caching=False)
+            if not args.eager:
+                runner.enable_decode_graphs(B, ctx + page, measure_products=False)
+            for lc in runner.layer_caches:
+                if lc.k is not None:
+                    lc.k.normal_(0, 1)
+                    lc.v.normal_(0, 1)
+            toks = torch.randint(0, DESIGN_VOCAB, (T,), generator=gen).tolist()
+            times = []
+            for r in range(5):
+                runner.cache.admit("p")
+                runner.cache.reserve("p", T)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                runner.step([StepEntry("p", toks, 0, [T - 1])])
+                torch.cuda.synchronize()
+                if r >= 2:
+                    times.append(time.perf_counter() - t0)
+                runner.cache.release("p")
+            pre_s = sum(times) / len(times)
+            steps, warmup = args.steps, args.warmup
+            start = ctx - (steps + warmup)
+            ids = [f"d{i}" for i in range(B)]
+            for rid in ids:
+                runner.cache.admit(rid)
+                runner.cache.reserve(rid, start)
+            tok = torch.randint(0, DESIGN_VOCAB, (B,), generator=gen).tolist()
+            t0 = None
+            for i in range(warmup + steps):
+                if i == warmup:
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                entries = []
+                for rid, t in zip(ids, tok):
+                    runner.cache.reserve(rid, start + i + 1)
+                    entries.append(StepEntry(rid, [t], start + i, [0]))
+                runner.step(entries)
+            torch.cuda.synchronize()
+            dec_s = (time.perf_counter() - t0) / steps
+            for rid in ids:
+                runner.cache.release(rid)
+            kernels.check_faults()
+            out[width][name] = {"prefill_tok_s": round(T / pre_s, 1), "prefill_ms": round(pre_s * 1e3, 3),
+                                "decode_tok_s": round(B / dec_s, 1), "decode_ms_per_step": round(dec_s * 1e3, 4)}
+            print(f"# width {width} {name}: prefill {T} tokens {pre_s * 1e3:.2f} ms, decode batch {B} context {ctx} "
+                  f"{dec_s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+            del runner, model
+            torch.cuda.empty_cache()
+    first = out[next(iter(out))]
+    line = {"metric": f"--design {args.design}: prefill tok/s @ {T} tokens and decode tok/s @ batch {B}, context {ctx}, "
+                      f"{layers} layers, beside Qwen3 at equal layer sizes",
+            "value": first[args.design]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": first[args.design]["decode_ms_per_step"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic", "config": {"model": f"{args.design} and qwen3, random weights", "global_batch": B,
+                                            "seq_len": ctx, "parallelism": "single GPU", "layers": layers,
+                                            "vocab_size": DESIGN_VOCAB, "decode_graph": not args.eager},
+            "designs": {str(w): v for w, v in out.items()}}
+    print(json.dumps(line), flush=True)
+    return 0
 
 
 def serve_run(args, config_json):
@@ -90,6 +208,8 @@ def main():
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not measured")
         return 2
+    if args.design:
+        return design_run(args)
 
     import torch
     from nano_vllm_amd.config import EngineConfig, Qwen3Config
