@@ -189,7 +189,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
                    const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
                    const int32_t* __restrict__ block_tables, int table_stride, int tokens, int max_segments,
                    int num_q_heads, int num_kv_heads, int page_size, float scale, int window,
-                   int32_t* error_flag) {
+                   const float* __restrict__ sinks, int32_t* error_flag) {
     constexpr int KP = D / 32;          // 16-byte pieces of a key row per lane = MFMAs per S tile
     constexpr int DT = D / 16;          // 16-channel tiles of the output
     const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
@@ -351,6 +351,8 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
     if (col < G) {
         const int head = kvh * G + col;
         if (rec.w == 1) {
+            // a sink: one more term exp(sink) in the denominator, in the units of the running maximum
+            if (sinks) l_run += __builtin_amdgcn_exp2f(sinks[head] * 1.4426950408889634f - fmaxf(m_run, -1e30f) * c_exp);
             const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
             __bf16* orow = out + t * out_stride + (int64_t)head * D;
 #pragma unroll
@@ -397,7 +399,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
 __global__ void __launch_bounds__(MERGE_WAVES * NVA_WAVE)
 attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                          const int32_t* __restrict__ plan, __bf16* __restrict__ out, int64_t out_stride,
-                         int num_q_heads, int head_dim) {
+                         int num_q_heads, int head_dim, const float* __restrict__ sinks) {
     __shared__ float acc_s[MERGE_WAVES][4 * NVA_WAVE];
     __shared__ float l_s[MERGE_WAVES];
     const int64_t t = blockIdx.x;
@@ -438,6 +440,7 @@ attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restri
     l = 0.f;
 #pragma unroll
     for (int w = 0; w < MERGE_WAVES; ++w) l += l_s[w];
+    if (sinks) l += __expf(sinks[head] - m);              // the sink joins the denominator once, after the segments
     const float inv = l > 0.f ? 1.f / l : 0.f;
     __bf16* orow = out + t * out_stride + (int64_t)head * head_dim;
 #pragma unroll
@@ -455,7 +458,7 @@ attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restri
 __global__ void __launch_bounds__(MERGE_WAVES * NVA_WAVE)
 attn_decode_merge_wave_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                               const int32_t* __restrict__ plan, __bf16* __restrict__ out, int64_t out_stride,
-                              int tokens, int num_q_heads, int head_dim) {
+                              int tokens, int num_q_heads, int head_dim, const float* __restrict__ sinks) {
     const int lane = threadIdx.x % NVA_WAVE;
     const int64_t pair = (int64_t)blockIdx.x * MERGE_WAVES + threadIdx.x / NVA_WAVE;
     if (pair >= (int64_t)tokens * num_q_heads) return;
@@ -489,6 +492,7 @@ attn_decode_merge_wave_kernel(const float* __restrict__ part_o, const float* __r
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[i] += v[j][i] * wj[j];
     }
+    if (sinks) l += __expf(sinks[head] - m);
     const float inv = l > 0.f ? 1.f / l : 0.f;
     __bf16* orow = out + t * out_stride + (int64_t)head * head_dim;
 #pragma unroll
@@ -587,12 +591,14 @@ NVA_EXPORT int nva_attn_decode_plan_bf16(const int32_t* positions, const int32_t
 
 // Refuses (non-zero code and a message) shapes this kernel does not take: the host wrapper checks
 // the same limits first and runs the general kernel for them.  plan: made by nva_attn_decode_plan for these tokens, kv heads, page size and
-// window; max_segments and waves from nva_attn_decode_plan_size.
+// window; max_segments and waves from nva_attn_decode_plan_size.  sinks, float [heads] or null: exp(sink_h)
+// joins the denominator of head h's softmax once (a key without a value).
 NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride, float* scratch,
                                     const int32_t* plan, const void* k_cache, const void* v_cache,
                                     const int32_t* block_tables, int table_stride, int64_t tokens, int num_q_heads,
                                     int num_kv_heads, int head_dim, int page_size, float scale, int window,
-                                    int max_segments, int waves, int32_t* error_flag, hipStream_t stream) {
+                                    int max_segments, int waves, const float* sinks, int32_t* error_flag,
+                                    hipStream_t stream) {
     if (tokens == 0) return 0;
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
         return nva_fail("attn_decode: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
@@ -620,7 +626,7 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     hipLaunchKernelGGL(attn_decode_kernel<DD>, dim3((unsigned)waves), dim3(NVA_WAVE), 0, stream, (const __bf16*)q, \
                        q_stride, (__bf16*)out, out_stride, part_o, part_ml, plan, (const __bf16*)k_cache,         \
                        (const __bf16*)v_cache, block_tables, table_stride, (int)tokens, max_segments, num_q_heads,  \
-                       num_kv_heads, page_size, scale, window, error_flag)
+                       num_kv_heads, page_size, scale, window, sinks, error_flag)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;
@@ -641,12 +647,12 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     if (pairs >= 2 * resident) {            // pairs enough for a wave each
         hipLaunchKernelGGL(attn_decode_merge_wave_kernel, dim3((unsigned)((pairs + MERGE_WAVES - 1) / MERGE_WAVES)),
                            dim3(MERGE_WAVES * NVA_WAVE), 0, stream, part_o, part_ml, plan, (__bf16*)out, out_stride,
-                           (int)tokens, num_q_heads, head_dim);
+                           (int)tokens, num_q_heads, head_dim, sinks);
         return nva_check_launch("attn_decode_merge");
     }
     dim3 mgrid((unsigned)tokens, (unsigned)num_q_heads);
     hipLaunchKernelGGL(attn_decode_merge_kernel, mgrid, dim3(MERGE_WAVES * NVA_WAVE), 0, stream, part_o, part_ml, plan,
-                       (__bf16*)out, out_stride, num_q_heads, head_dim);
+                       (__bf16*)out, out_stride, num_q_heads, head_dim, sinks);
     return nva_check_launch("attn_decode_merge");
 }
 

@@ -93,7 +93,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
                     const int32_t* __restrict__ block_tables, int table_stride,
                     const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ kv_lens,
                     const int32_t* __restrict__ tiles, int num_tiles, int paired, int num_q_heads, int num_kv_heads,
-                    int page_size, float scale, int window, int32_t* error_flag) {
+                    int page_size, float scale, int window, const float* __restrict__ sinks, int32_t* error_flag) {
     constexpr int DC = D / 16;            // 16-channel steps of the first product
     constexpr int MT = D / 32;            // 32-channel tiles of the output
     constexpr int KR = D / 8;             // 16-byte pieces of a K row (one key)
@@ -506,10 +506,14 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[mt][e] = acc[mt][e] * f_own + share[(mt * 16 + e) * NVA_WAVE] * f_other;
+        m_run = fmaxf(m_run, m_other);       // what sum and accumulators now refer to
     }
 
     // acc[mt][4a + b] = O[query col][channel 32*mt + 8a + 4h + b]
     if (!active || !row_ok) return;
+    // a sink: one more term exp(sink) in the denominator (a key without a value), in the units of the
+    // running maximum; it joins once, after the tiles (and after the sets of waves have met)
+    if (sinks) l_run += __builtin_amdgcn_exp2f(sinks[head] * 1.4426950408889634f - fmaxf(m_run, -1e30f) * c_exp);
     const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
     __bf16* orow = out + (int64_t)(q_begin + row) * out_stride + (int64_t)head * D;
 #pragma unroll
@@ -536,7 +540,7 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
                                      int table_stride, const int32_t* cu_seqlens_q, const int32_t* kv_lens,
                                      const int32_t* tiles, int64_t num_tiles, int num_q_heads,
                                      int num_kv_heads, int head_dim, int page_size, float scale, int window,
-                                     int32_t* error_flag, hipStream_t stream) {
+                                     const float* sinks, int32_t* error_flag, hipStream_t stream) {
     if (num_tiles == 0) return 0;
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
         return nva_fail("attn_prefill: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
@@ -576,7 +580,7 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
                        (const __bf16*)q, q_stride, (__bf16*)out, out_stride, (const __bf16*)k_cache,                 \
                        (const __bf16*)v_cache, block_tables, table_stride, cu_seqlens_q, kv_lens, tiles,             \
                        (int)num_tiles, SS == 1 && PF_WAVES_PER_SIMD(DD) == 2 && total <= 2 * cus ? (int)total : 0,   \
-                       num_q_heads, num_kv_heads, page_size, scale, window, error_flag)
+                       num_q_heads, num_kv_heads, page_size, scale, window, sinks, error_flag)
 #define LAUNCH(DD)                                                                                                 \
     do {                                                                                                           \
         if (PF_WAVES_PER_SIMD(DD) == 2 && two_sets) LAUNCH_SETS(DD, PF_WAVES_PER_SIMD(DD));                         \

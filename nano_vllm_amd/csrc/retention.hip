@@ -135,6 +135,178 @@ retention_chunk_kernel(const T* __restrict__ proj, int64_t stride, float* __rest
     }
 }
 
+// ---------------------------------------------------------------------------- on the matrix cores, in float
+// The same chunks with their four products as 32 x 32 x 2 float MFMAs (float operands, float sums:
+// nothing is rounded to a shorter type).  One wave per (request, head, 32 value channels), up to four
+// waves of one head in a workgroup, which share the chunk's q and k in LDS; heads of 32 DT channels.
+// The wave keeps its part of the state, S[:, 32 channels], in DT accumulator tiles
+// for the whole portion: it is the B operand of the product with q as it lies (register r of a tile
+// holds, in the lanes' lower and upper halves, rows 8 (r/4) + r%4 and that + 4, so step r of the sum
+// over a tile's 32 rows takes these two rows, and q is read from LDS to match), and the accumulator
+// of the product k^T v.  Per chunk: scores q k^T (DT * 16 MFMAs), masked and weighted by the decay
+// powers and passed through LDS to become an A operand; o = scores v + decay^(i+1) q S (16 + DT * 16);
+// S <- decay^n S + k^T (decay^(n-1-j) v) (DT * 16).  Rows of a short chunk beyond its n tokens are zero.
+// cos_sin: float [tokens, rot], cosines then sines of each token's angles (made once per step by
+// retention_angles_kernel, with the accurate routines), or null where nothing is rotated.
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+__global__ void __launch_bounds__(256)
+retention_angles_kernel(const int32_t* __restrict__ positions, const float* __restrict__ inv_freq, int half,
+                        float* __restrict__ cos_sin, int64_t total) {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= total) return;
+    const int64_t t = e / half;
+    const int i = (int)(e % half);
+    float sn, cs;
+    sincosf((float)positions[t] * inv_freq[i], &sn, &cs);
+    cos_sin[t * 2 * half + i] = cs;
+    cos_sin[t * 2 * half + half + i] = sn;
+}
+
+#define RET_MFMA_WAVES 4
+__host__ __device__ inline size_t ret_mfma_lds_floats(int dim, int waves) {
+    return (size_t)2 * RET_C * (dim + 1) + (size_t)waves * 2 * RET_C * (RET_C + 1) + 64;
+}
+
+template <typename T, int DT>
+__global__ void __launch_bounds__(RET_MFMA_WAVES * NVA_WAVE)
+retention_mfma_kernel(const T* __restrict__ proj, int64_t stride, float* __restrict__ o_raw, int64_t o_stride,
+                      float* __restrict__ state, const int32_t* __restrict__ cu_seqlens_q,
+                      const int32_t* __restrict__ seq_starts, const int32_t* __restrict__ state_slots,
+                      const float* __restrict__ decay_pow, const float* __restrict__ cos_sin, int rot,
+                      int heads, int vdim, float k_scale) {
+    static_assert(RET_C == 32, "a chunk is one MFMA tile of rows");
+    constexpr int D = 32 * DT, DS = D + 1, VS = RET_C + 1;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int waves = blockDim.x / NVA_WAVE, wave = threadIdx.x / NVA_WAVE;
+    float* const q_s = lds;                                   // [32][DS], all waves'
+    float* const k_s = q_s + RET_C * DS;                      // [32][DS]
+    float* const pw_s = k_s + RET_C * DS;                     // [33] (+ padding to 64)
+    float* const v_s = pw_s + 64 + wave * 2 * RET_C * VS;     // [32][33], this wave's
+    float* const a_s = v_s + RET_C * VS;                      // [32][33]
+
+    const int lane = threadIdx.x % NVA_WAVE, col = lane & 31, up = lane >> 5;
+    const int nslices = vdim / 32, groups = (nslices + waves - 1) / waves;
+    const int h = blockIdx.x / groups;
+    const int slice = (blockIdx.x % groups) * waves + wave;
+    const bool active = slice < nslices;                      // a wave without a slice only helps to load q and k
+    const int c0 = 32 * (active ? slice : 0);
+    const int seq = blockIdx.y;
+    const int q_begin = cu_seqlens_q[seq];
+    const int q_len = cu_seqlens_q[seq + 1] - q_begin;
+    const int start = seq_starts[seq];
+    const int slot = state_slots[seq];
+    float* const s_g = state + (((int64_t)slot * heads + h) * D) * vdim + c0 + col;
+    const int half = rot / 2;
+    const int64_t q_off = (int64_t)h * D, k_off = (int64_t)(heads + h) * D;
+    const int64_t v_off = (int64_t)2 * heads * D + (int64_t)h * vdim + c0;
+    // register r of an accumulator tile holds row rowmap(r) of the tile in this lane's half of the wave
+    auto rowmap = [&](int r) { return 8 * (r >> 2) + 4 * up + (r & 3); };
+
+    if (threadIdx.x <= RET_C) pw_s[threadIdx.x] = decay_pow[(int64_t)h * (RET_C + 1) + threadIdx.x];
+    f32x16 S[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) S[dt][r] = start > 0 && active ? s_g[(int64_t)(32 * dt + rowmap(r)) * vdim] : 0.f;
+
+    for (int t0 = 0; t0 < q_len; t0 += RET_C) {
+        const int n = min(RET_C, q_len - t0);
+        __syncthreads();                          // the chunk before is done with LDS
+        for (int e = threadIdx.x; e < RET_C * D; e += blockDim.x) {
+            const int r = e / D, d = e % D;
+            float qv = 0.f, kv = 0.f;
+            if (r < n) {
+                const int64_t tok = q_begin + t0 + r;
+                const T* row = proj + tok * stride;
+                qv = to_float(row[q_off + d]);
+                kv = to_float(row[k_off + d]);
+                if (d < rot) {
+                    const bool lower = d < half;
+                    const int partner = lower ? d + half : d - half;
+                    const float* cs_row = cos_sin + tok * rot;
+                    const float cs = cs_row[lower ? d : d - half], sn = cs_row[half + (lower ? d : d - half)];
+                    const float qp = to_float(row[q_off + partner]), kp = to_float(row[k_off + partner]);
+                    qv = lower ? qv * cs - qp * sn : qv * cs + qp * sn;
+                    kv = lower ? kv * cs - kp * sn : kv * cs + kp * sn;
+                }
+            }
+            q_s[r * DS + d] = qv;
+            k_s[r * DS + d] = kv * k_scale;
+        }
+        for (int e = lane; e < RET_C * 32; e += NVA_WAVE) {
+            const int r = e >> 5, c = e & 31;
+            v_s[r * VS + c] = r < n ? to_float(proj[(int64_t)(q_begin + t0 + r) * stride + v_off + c]) : 0.f;
+        }
+        __syncthreads();
+        // ---- scores: A[i][j] = q_i . k_j
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        {
+            const float* qa = q_s + col * DS + up;
+            const float* kb = k_s + col * DS + up;
+#pragma unroll 8
+            for (int kk = 0; kk < D / 2; ++kk)
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[2 * kk], kb[2 * kk], acc, 0, 0, 0);
+        }
+        // masked and weighted by the decay's powers, then through LDS to become an A operand
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int i = rowmap(r);
+            a_s[i * VS + col] = col <= i ? acc[r] * pw_s[i - col] : 0.f;
+        }
+        __syncthreads();
+        // ---- outputs: o = A v + decay^(i+1) q S
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        {
+            const float* aa = a_s + col * VS + up;
+            const float* vb = v_s + up * VS + col;
+#pragma unroll
+            for (int kk = 0; kk < RET_C / 2; ++kk)
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(aa[2 * kk], vb[2 * kk * VS], acc, 0, 0, 0);
+            const float row_decay = pw_s[col + 1];
+            const float* qa = q_s + col * DS + 4 * up;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[32 * dt + 8 * (r >> 2) + (r & 3)] * row_decay, S[dt][r],
+                                                               acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int i = rowmap(r);
+            if (i < n && active) o_raw[(int64_t)(q_begin + t0 + i) * o_stride + (int64_t)h * vdim + c0 + col] = acc[r];
+        }
+        // ---- the state after the chunk: S <- decay^n S + k^T (decay^(n-1-j) v)
+        {
+            const float all = pw_s[n];
+            float vb[RET_C / 2];
+#pragma unroll
+            for (int kk = 0; kk < RET_C / 2; ++kk) {
+                const int j = 2 * kk + up;
+                vb[kk] = j < n ? v_s[j * VS + col] * pw_s[n - 1 - j] : 0.f;
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) S[dt][r] *= all;
+                const float* ka = k_s + up * DS + 32 * dt + col;
+#pragma unroll
+                for (int kk = 0; kk < RET_C / 2; ++kk)
+                    S[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[2 * kk * DS], vb[kk], S[dt], 0, 0, 0);
+            }
+        }
+    }
+    if (!active) return;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s_g[(int64_t)(32 * dt + rowmap(r)) * vdim] = S[dt][r];
+}
+
 // y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * silu(g[t, h, :]); one wave per (token, head).
 template <typename T>
 __global__ void __launch_bounds__(NVA_WAVE)
@@ -159,12 +331,14 @@ retention_finish_kernel(const float* __restrict__ o_raw, int64_t o_stride, const
 // o_raw: float [tokens, heads * vdim] scratch.  y: [tokens, heads * vdim] elements.
 // state: float [slots, heads, dim, vdim].  decay_pow: float [heads, RET_C + 1], decay_h^m.
 // inv_freq: float [rot / 2] (rot 0: no rotation).  vslice: value channels per workgroup (1..32).
+// matrix_cores != 0: heads of a multiple of 32 channels (up to 256) and values of a multiple of 32 run
+// the MFMA kernel, which wants the tokens' positions and float [tokens, rot] of scratch for the angles.
 NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* o_raw, void* y, int64_t y_stride,
                                        float* state, int64_t num_slots, const int32_t* cu_seqlens_q,
                                        const int32_t* seq_starts, const int32_t* state_slots, int64_t num_seqs,
                                        int64_t tokens, const float* decay_pow, const float* inv_freq, int rot,
                                        int heads, int dim, int vdim, int vslice, float k_scale, float eps,
-                                       hipStream_t stream) {
+                                       const int32_t* positions, float* cos_sin, int matrix_cores, hipStream_t stream) {
     if (num_seqs == 0 || tokens == 0) return 0;
     if (num_seqs < 0 || num_seqs > 65535 || tokens < 0 || tokens > 0x7fffffff)
         return nva_fail("retention: bad counts requests=%lld tokens=%lld", (long long)num_seqs, (long long)tokens);
@@ -176,6 +350,51 @@ NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* 
     if (stride < width || y_stride < (int64_t)heads * vdim) return nva_fail("retention: rows are too short");
     if (!proj || !o_raw || !y || !state || !cu_seqlens_q || !seq_starts || !state_slots || !decay_pow || num_slots <= 0)
         return nva_fail("retention: a needed tensor is missing");
+    const elem_t* p = (const elem_t*)proj;
+    if (matrix_cores && dim % 32 == 0 && dim <= 256 && vdim % 32 == 0) {
+        // positions: int32 [tokens]; cos_sin: float [tokens, rot] scratch (both needed with a rotation)
+        if (rot && (!positions || !cos_sin)) return nva_fail("retention: the rotation needs positions and room for the angles");
+        if (rot) {
+            const int64_t total = tokens * (rot / 2);
+            hipLaunchKernelGGL(retention_angles_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, positions,
+                               inv_freq, rot / 2, cos_sin, total);
+        }
+        const int nsl = vdim / 32;
+        const int waves = nsl < RET_MFMA_WAVES ? nsl : RET_MFMA_WAVES;
+        const int groups = (nsl + waves - 1) / waves;
+        const size_t bytes = ret_mfma_lds_floats(dim, waves) * sizeof(float);
+        dim3 grid((unsigned)(heads * groups), (unsigned)num_seqs);
+#define RET_LAUNCH(DTT)                                                                                             \
+        {                                                                                                           \
+            auto kernel = retention_mfma_kernel<elem_t, DTT>;                                                        \
+            static bool raised = false;                                                                              \
+            if (!raised && bytes > 48 * 1024) {                                                                       \
+                if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) \
+                    return nva_fail("retention: cannot have %zu bytes of LDS", bytes);                               \
+                raised = true;                                                                                       \
+            }                                                                                                        \
+            hipLaunchKernelGGL(kernel, grid, dim3(waves * NVA_WAVE), bytes, stream, p, stride, o_raw,               \
+                               (int64_t)heads * vdim, state, cu_seqlens_q, seq_starts, state_slots, decay_pow, cos_sin, \
+                               rot, heads, vdim, k_scale);                                                           \
+        }
+        switch (dim / 32) {
+            case 1: RET_LAUNCH(1); break;
+            case 2: RET_LAUNCH(2); break;
+            case 3: RET_LAUNCH(3); break;
+            case 4: RET_LAUNCH(4); break;
+            case 5: RET_LAUNCH(5); break;
+            case 6: RET_LAUNCH(6); break;
+            case 7: RET_LAUNCH(7); break;
+            default: RET_LAUNCH(8); break;
+        }
+#undef RET_LAUNCH
+        int rc = nva_check_launch("retention (matrix cores)");
+        if (rc) return rc;
+        const elem_t* gate = p + (int64_t)2 * heads * dim + (int64_t)heads * vdim;
+        hipLaunchKernelGGL((retention_finish_kernel<elem_t>), dim3((unsigned)tokens, (unsigned)heads), dim3(NVA_WAVE), 0,
+                           stream, o_raw, (int64_t)heads * vdim, gate, stride, (elem_t*)y, y_stride, vdim, eps);
+        return nva_check_launch("retention_finish");
+    }
     const int nslices = (vdim + vslice - 1) / vslice;
     if ((int64_t)heads * nslices > 0x7fffffff) return nva_fail("retention: too many workgroups");
     const size_t lds = ret_lds_floats(dim, vslice) * sizeof(float);
@@ -187,7 +406,6 @@ NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* 
             return nva_fail("retention: cannot have %zu bytes of LDS", lds);
         raised = 160 * 1024;
     }
-    const elem_t* p = (const elem_t*)proj;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(heads * nslices), (unsigned)num_seqs), dim3(RET_THREADS), lds, stream, p,
                        stride, o_raw, (int64_t)heads * vdim, state, cu_seqlens_q, seq_starts, state_slots, decay_pow,
                        inv_freq, rot, heads, dim, vdim, vslice, nslices, k_scale);

@@ -252,6 +252,8 @@ class HipKernels:
         self.fuse_split_sums = True         # False: every product is finished by its own pass
         # False: attention always runs the general kernel (tests compare the two)
         self.mfma_attention = True
+        # False: retention always runs the general kernel
+        self.mfma_retention = True
         # False: the general kernel runs one wave per token for portions of prompts too (the same bits, slower)
         self.tiled_general_attention = True
 
@@ -966,13 +968,12 @@ class HipKernels:
         # them where its shape limits allow; everything else runs the general kernel
         start = 0
         # (the matrix-core kernels fold the scale into the exponent, which needs it positive)
-        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and \
-            v_dim == head_dim and sinks is None
+        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim
         if batch.num_decode > 0 and mfma and \
                 self._decode_kernel_takes(num_heads // num_kv_heads, head_dim, page_size, q, qs, out, os_):
             start = batch.num_decode
             self._attention_decode(q, qs, out, os_, k_cache, v_cache, tables, batch, start, num_heads, num_kv_heads,
-                                   head_dim, page_size, scale, window)
+                                   head_dim, page_size, scale, window, sinks)
         if start < tokens and mfma and start == batch.num_decode and \
                 self._prefill_kernel_takes(head_dim, page_size, tables.shape[1], q, qs, out, os_):
             # portions of prompts: the matrix-core prefill kernel, one workgroup per 32 query rows
@@ -981,7 +982,7 @@ class HipKernels:
                          _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.cu_seqlens_q), _p(batch.kv_lens),
                          _p(tiles), c_i64(tiles.shape[0]), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
-                         _p(self.fault_flag), self._stream())
+                         _p(sinks), _p(self.fault_flag), self._stream())
             start = tokens
         if self.tiled_general_attention and start <= batch.num_decode < tokens and not window and \
                 max(head_dim, v_dim) <= GENERAL_TILED_MAX_HEAD_DIM:
@@ -1050,10 +1051,16 @@ class HipKernels:
         while vslice > 8 and seqs * heads * ((v_dim + vslice - 1) // vslice) < self.cus:
             vslice //= 2
         vslice = min(vslice, max(1, v_dim))
+        positions = scratch = None
+        if self.mfma_retention and rot and dim % 32 == 0 and dim <= 256 and v_dim % 32 == 0:
+            _i32(batch.positions, tokens, "positions")
+            positions = batch.positions
+            scratch = torch.empty((tokens, rot), dtype=torch.float32, device=proj.device)
         library.call("retention", _suffix(proj), "nva_retention", _p(proj), c_i64(stride), _p(raw), _p(out), c_i64(os_),
                      _p(state), c_i64(state.shape[0]), _p(batch.cu_seqlens_q), _p(batch.seq_starts),
                      _p(batch.state_slots), c_i64(seqs), c_i64(tokens), _p(decay_powers), _p(inv_freq), c_i32(rot),
-                     c_i32(heads), c_i32(dim), c_i32(v_dim), c_i32(vslice), c_f32(k_scale), c_f32(eps), self._stream())
+                     c_i32(heads), c_i32(dim), c_i32(v_dim), c_i32(vslice), c_f32(k_scale), c_f32(eps), _p(positions),
+                     _p(scratch), c_i32(1 if self.mfma_retention else 0), self._stream())
         return out
 
     @staticmethod
@@ -1097,7 +1104,7 @@ class HipKernels:
                                                                              out_stride)
 
     def _attention_decode(self, q, qs, out, os_, k_cache, v_cache, tables, batch, n, num_heads, num_kv_heads,
-                          head_dim, page_size, scale, window):
+                          head_dim, page_size, scale, window, sinks=None):
         # The work is shared out on the device from the tokens' positions, once per step and (kv
         # heads, window): the first layer that asks makes the plan, the others find it on the batch.
         # The library says how large the partial results may get for this many tokens of at most
@@ -1125,7 +1132,7 @@ class HipKernels:
                          _p(scratch), _p(plan), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
                          c_i64(t1 - t0), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
-                         c_i32(bound), c_i32(waves), _p(self.fault_flag), self._stream())
+                         c_i32(bound), c_i32(waves), _p(sinks), _p(self.fault_flag), self._stream())
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:

@@ -82,7 +82,7 @@ class Attention(Part):
     @property
     def kernel_modules(self):
         prepare = "qk_rownorm" if self.row_prepare else "rope"
-        if self.sink or self.v_head_dim != self.head_dim:
+        if self.v_head_dim != self.head_dim:
             return (prepare, "attn_generic")
         return (prepare, "attn_generic", "attn_decode", "attn_prefill")
 

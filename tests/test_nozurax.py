@@ -300,6 +300,7 @@ def _plain_retention_of_projections(proj, heads, dim, vdim, decay, rot, base, ep
 def _state_batch(dev, q_lens, starts, slots):
     return SimpleNamespace(
         num_seqs=len(q_lens), q_lens=list(q_lens), starts=list(starts),
+        positions=torch.tensor([p for s, n in zip(starts, q_lens) for p in range(s, s + n)], dtype=torch.int32, device=dev),
         cu_seqlens_q=torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32, device=dev),
         seq_starts=torch.tensor(starts, dtype=torch.int32, device=dev),
         state_slots=torch.tensor(slots, dtype=torch.int32, device=dev))
@@ -322,6 +323,11 @@ def _retention_constants(k, dev, decay, dim, rot, base):
     (2, 24, 40, (0.97, 1.0), 0, 0.0),
     (2, 64, 72, (0.96875, 0.998), 64, 1e4),
     (2, 6, 10, (0.0, 0.99), 4, 50.0),
+    # heads and values of multiples of 32 channels: the kernel on the matrix cores
+    (2, 64, 64, (0.96875, 0.998), 64, 1e4),
+    (2, 128, 160, (0.9, 0.999), 64, 1e6),
+    (1, 256, 32, (0.99,), 0, 0.0),
+    (3, 96, 96, (0.5, 1.0, 0.75), 96, 100.0),
 ])
 def test_retention_in_portions_of_every_size_and_token_by_token(backend, dtype, heads, dim, vdim, decay, rot, base):
     k, dev = _kernels(backend, dtype)
