@@ -135,6 +135,73 @@ retention_chunk_kernel(const T* __restrict__ proj, int64_t stride, float* __rest
     }
 }
 
+// ---------------------------------------------------------------------------- single tokens
+// A request that brings one token: S <- decay S + k v^T, o = S^T q, nothing else.  The step is the
+// state's bytes, read once and written once: a workgroup takes (request, head, 32 value channels),
+// a thread one channel and every eighth row of S, which it asks for before anything else; q and k
+// are rotated into LDS meanwhile, and the eight partial sums of a channel meet in LDS.
+#define RET_DEC_ROWS 32           // rows of S a thread keeps: heads of up to 8 * 32 channels
+template <typename T>
+__global__ void __launch_bounds__(256)
+retention_decode_kernel(const T* __restrict__ proj, int64_t stride, float* __restrict__ o_raw, int64_t o_stride,
+                        float* __restrict__ state, const int32_t* __restrict__ cu_seqlens_q,
+                        const int32_t* __restrict__ seq_starts, const int32_t* __restrict__ state_slots,
+                        const float* __restrict__ decay_pow, const float* __restrict__ inv_freq, int rot,
+                        int heads, int dim, int vdim, int nslices, float k_scale) {
+    __shared__ float q_s[8 * RET_DEC_ROWS], k_s[8 * RET_DEC_ROWS], part_s[8][33];
+    const int h = blockIdx.x / nslices, c0 = 32 * (blockIdx.x % nslices);
+    const int seq = blockIdx.y;
+    const int tid = threadIdx.x, c = tid & 31, dg = tid >> 5;
+    const bool has = c0 + c < vdim;
+    const int64_t tok = cu_seqlens_q[seq];
+    const int start = seq_starts[seq];
+    const int slot = state_slots[seq];
+    float* const s_g = state + (((int64_t)slot * heads + h) * dim) * vdim + c0 + c;
+    float S[RET_DEC_ROWS];
+#pragma unroll
+    for (int i = 0; i < RET_DEC_ROWS; ++i) {
+        const int d = dg + 8 * i;
+        S[i] = has && d < dim && start > 0 ? s_g[(int64_t)d * vdim] : 0.f;
+    }
+    const T* row = proj + tok * stride;
+    const int half = rot / 2;
+    for (int d = tid; d < dim; d += blockDim.x) {
+        float qv = to_float(row[(int64_t)h * dim + d]), kv = to_float(row[(int64_t)(heads + h) * dim + d]);
+        if (d < rot) {
+            const bool lower = d < half;
+            const int partner = lower ? d + half : d - half;
+            float sn, cs;
+            sincosf((float)start * inv_freq[lower ? d : d - half], &sn, &cs);
+            const float qp = to_float(row[(int64_t)h * dim + partner]), kp = to_float(row[(int64_t)(heads + h) * dim + partner]);
+            qv = lower ? qv * cs - qp * sn : qv * cs + qp * sn;
+            kv = lower ? kv * cs - kp * sn : kv * cs + kp * sn;
+        }
+        q_s[d] = qv;
+        k_s[d] = kv * k_scale;
+    }
+    const float v = has ? to_float(row[(int64_t)2 * heads * dim + (int64_t)h * vdim + c0 + c]) : 0.f;
+    const float decay = decay_pow[(int64_t)h * (RET_C + 1) + 1];
+    __syncthreads();
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < RET_DEC_ROWS; ++i) {
+        const int d = dg + 8 * i;
+        if (d < dim) {
+            S[i] = decay * S[i] + k_s[d] * v;
+            o += S[i] * q_s[d];
+            if (has) s_g[(int64_t)d * vdim] = S[i];
+        }
+    }
+    part_s[dg][c] = o;
+    __syncthreads();
+    if (dg == 0 && has) {
+        float sum = 0.f;
+#pragma unroll
+        for (int g = 0; g < 8; ++g) sum += part_s[g][c];
+        o_raw[tok * o_stride + (int64_t)h * vdim + c0 + c] = sum;
+    }
+}
+
 // ---------------------------------------------------------------------------- on the matrix cores, in float
 // The same chunks with their four products as 32 x 32 x 2 float MFMAs (float operands, float sums:
 // nothing is rounded to a shorter type).  One wave per (request, head, 32 value channels), up to four
@@ -164,21 +231,44 @@ retention_angles_kernel(const int32_t* __restrict__ positions, const float* __re
 }
 
 #define RET_MFMA_WAVES 4
+
+// Eight consecutive elements as they were loaded (16 bytes of bfloat16, 32 of float), widened when used.
+template <typename T> struct Raw8;
+template <> struct Raw8<__bf16> {
+    typedef __attribute__((ext_vector_type(8))) __bf16 v8;
+    v8 v;
+    __device__ __forceinline__ void load(const __bf16* p) { v = *reinterpret_cast<const v8*>(p); }
+    __device__ __forceinline__ float get(int i) const { return static_cast<float>(v[i]); }
+};
+template <> struct Raw8<float> {
+    float4 a, b;
+    __device__ __forceinline__ void load(const float* p) {
+        a = reinterpret_cast<const float4*>(p)[0];
+        b = reinterpret_cast<const float4*>(p)[1];
+    }
+    __device__ __forceinline__ float get(int i) const {
+        return i == 0 ? a.x : i == 1 ? a.y : i == 2 ? a.z : i == 3 ? a.w : i == 4 ? b.x : i == 5 ? b.y : i == 6 ? b.z : b.w;
+    }
+};
+
 __host__ __device__ inline size_t ret_mfma_lds_floats(int dim, int waves) {
     return (size_t)2 * RET_C * (dim + 1) + (size_t)waves * 2 * RET_C * (RET_C + 1) + 64;
 }
 
-template <typename T, int DT>
-__global__ void __launch_bounds__(RET_MFMA_WAVES * NVA_WAVE)
+// NW: waves of the workgroup.  vec: rows, offsets and the rotation allow loads of eight elements; the
+// chunk after the one at hand is then asked for before the products start and waits in registers.
+template <typename T, int DT, int NW>
+__global__ void __launch_bounds__(NW * NVA_WAVE)
 retention_mfma_kernel(const T* __restrict__ proj, int64_t stride, float* __restrict__ o_raw, int64_t o_stride,
                       float* __restrict__ state, const int32_t* __restrict__ cu_seqlens_q,
                       const int32_t* __restrict__ seq_starts, const int32_t* __restrict__ state_slots,
                       const float* __restrict__ decay_pow, const float* __restrict__ cos_sin, int rot,
-                      int heads, int vdim, float k_scale) {
+                      int heads, int vdim, float k_scale, int vec) {
     static_assert(RET_C == 32, "a chunk is one MFMA tile of rows");
     constexpr int D = 32 * DT, DS = D + 1, VS = RET_C + 1;
     extern __shared__ __attribute__((aligned(16))) float lds[];
-    const int waves = blockDim.x / NVA_WAVE, wave = threadIdx.x / NVA_WAVE;
+    constexpr int waves = NW;
+    const int wave = threadIdx.x / NVA_WAVE;
     float* const q_s = lds;                                   // [32][DS], all waves'
     float* const k_s = q_s + RET_C * DS;                      // [32][DS]
     float* const pw_s = k_s + RET_C * DS;                     // [33] (+ padding to 64)
@@ -210,9 +300,83 @@ retention_mfma_kernel(const T* __restrict__ proj, int64_t stride, float* __restr
 #pragma unroll
         for (int r = 0; r < 16; ++r) S[dt][r] = start > 0 && active ? s_g[(int64_t)(32 * dt + rowmap(r)) * vdim] : 0.f;
 
+    // blocks of eight elements: of q and k [32][D / 8] over all threads, of v [32][4] over a wave's lanes
+    constexpr int QK_BLOCKS = RET_C * D / 8, PQ = (QK_BLOCKS + NW * NVA_WAVE - 1) / (NW * NVA_WAVE);
+    constexpr bool PREFETCH = PQ <= 4;
+    constexpr int PQR = PREFETCH ? PQ : 1;
+    Raw8<T> rq[PQR], rqp[PQR], rk[PQR], rkp[PQR], rv[2];
+    float4 rcs[PQR][2], rsn[PQR][2];
+    const bool fast = PREFETCH && vec;
+    auto ask = [&](int t0) __attribute__((always_inline)) {
+        const int n = min(RET_C, q_len - t0);
+#pragma unroll
+        for (int p = 0; p < PQR; ++p) {
+            const int b = threadIdx.x + p * NW * NVA_WAVE;
+            const int r = b / (D / 8), d = (b % (D / 8)) * 8;
+            if (b < QK_BLOCKS && r < n) {
+                const int64_t tok = q_begin + t0 + r;
+                const T* row = proj + tok * stride;
+                rq[p].load(row + q_off + d);
+                rk[p].load(row + k_off + d);
+                if (d < rot) {
+                    const int partner = d < half ? d + half : d - half, i0 = d < half ? d : d - half;
+                    rqp[p].load(row + q_off + partner);
+                    rkp[p].load(row + k_off + partner);
+                    const float* cs_row = cos_sin + tok * rot + i0;
+                    rcs[p][0] = reinterpret_cast<const float4*>(cs_row)[0];
+                    rcs[p][1] = reinterpret_cast<const float4*>(cs_row)[1];
+                    rsn[p][0] = reinterpret_cast<const float4*>(cs_row + half)[0];
+                    rsn[p][1] = reinterpret_cast<const float4*>(cs_row + half)[1];
+                }
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int b = lane + p * NVA_WAVE, r = b >> 2, c = (b & 3) * 8;
+            if (r < n) rv[p].load(proj + (int64_t)(q_begin + t0 + r) * stride + v_off + c);
+        }
+    };
+    auto put = [&](int n) __attribute__((always_inline)) {
+#pragma unroll
+        for (int p = 0; p < PQR; ++p) {
+            const int b = threadIdx.x + p * NW * NVA_WAVE;
+            const int r = b / (D / 8), d = (b % (D / 8)) * 8;
+            if (b < QK_BLOCKS) {
+                const bool lower = d < half;
+                const float cs[8] = {rcs[p][0].x, rcs[p][0].y, rcs[p][0].z, rcs[p][0].w, rcs[p][1].x, rcs[p][1].y, rcs[p][1].z, rcs[p][1].w};
+                const float sn[8] = {rsn[p][0].x, rsn[p][0].y, rsn[p][0].z, rsn[p][0].w, rsn[p][1].x, rsn[p][1].y, rsn[p][1].z, rsn[p][1].w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float qv = 0.f, kv = 0.f;
+                    if (r < n) {
+                        qv = rq[p].get(e), kv = rk[p].get(e);
+                        if (d < rot) {
+                            const float qp = rqp[p].get(e), kp = rkp[p].get(e);
+                            qv = lower ? qv * cs[e] - qp * sn[e] : qv * cs[e] + qp * sn[e];
+                            kv = lower ? kv * cs[e] - kp * sn[e] : kv * cs[e] + kp * sn[e];
+                        }
+                    }
+                    q_s[r * DS + d + e] = qv;
+                    k_s[r * DS + d + e] = kv * k_scale;
+                }
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int b = lane + p * NVA_WAVE, r = b >> 2, c = (b & 3) * 8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v_s[r * VS + c + e] = r < n ? rv[p].get(e) : 0.f;
+        }
+    };
+    if (fast) ask(0);
+
     for (int t0 = 0; t0 < q_len; t0 += RET_C) {
         const int n = min(RET_C, q_len - t0);
         __syncthreads();                          // the chunk before is done with LDS
+        if (fast) {
+            put(n);
+            if (t0 + RET_C < q_len) ask(t0 + RET_C);      // on its way during this chunk's products
+        } else {
         for (int e = threadIdx.x; e < RET_C * D; e += blockDim.x) {
             const int r = e / D, d = e % D;
             float qv = 0.f, kv = 0.f;
@@ -237,6 +401,7 @@ retention_mfma_kernel(const T* __restrict__ proj, int64_t stride, float* __restr
         for (int e = lane; e < RET_C * 32; e += NVA_WAVE) {
             const int r = e >> 5, c = e & 31;
             v_s[r * VS + c] = r < n ? to_float(proj[(int64_t)(q_begin + t0 + r) * stride + v_off + c]) : 0.f;
+        }
         }
         __syncthreads();
         // ---- scores: A[i][j] = q_i . k_j
@@ -338,7 +503,8 @@ NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* 
                                        const int32_t* seq_starts, const int32_t* state_slots, int64_t num_seqs,
                                        int64_t tokens, const float* decay_pow, const float* inv_freq, int rot,
                                        int heads, int dim, int vdim, int vslice, float k_scale, float eps,
-                                       const int32_t* positions, float* cos_sin, int matrix_cores, hipStream_t stream) {
+                                       const int32_t* positions, float* cos_sin, int matrix_cores, int64_t num_decode,
+                                       hipStream_t stream) {
     if (num_seqs == 0 || tokens == 0) return 0;
     if (num_seqs < 0 || num_seqs > 65535 || tokens < 0 || tokens > 0x7fffffff)
         return nva_fail("retention: bad counts requests=%lld tokens=%lld", (long long)num_seqs, (long long)tokens);
@@ -351,6 +517,25 @@ NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* 
     if (!proj || !o_raw || !y || !state || !cu_seqlens_q || !seq_starts || !state_slots || !decay_pow || num_slots <= 0)
         return nva_fail("retention: a needed tensor is missing");
     const elem_t* p = (const elem_t*)proj;
+    const elem_t* gate = p + (int64_t)2 * heads * dim + (int64_t)heads * vdim;
+    // The first num_decode requests bring one token each (the caller puts them first): their kernel
+    // streams the state; the portions after them run in chunks.
+    if (num_decode < 0 || num_decode > num_seqs) return nva_fail("retention: %lld single tokens of %lld requests", (long long)num_decode, (long long)num_seqs);
+    if (num_decode > 0 && dim <= 8 * RET_DEC_ROWS) {
+        const int nsl = (vdim + 31) / 32;
+        hipLaunchKernelGGL((retention_decode_kernel<elem_t>), dim3((unsigned)(heads * nsl), (unsigned)num_decode), dim3(256), 0,
+                           stream, p, stride, o_raw, (int64_t)heads * vdim, state, cu_seqlens_q, seq_starts, state_slots,
+                           decay_pow, inv_freq, rot, heads, dim, vdim, nsl, k_scale);
+        int rc = nva_check_launch("retention (single tokens)");
+        if (rc) return rc;
+        cu_seqlens_q += num_decode, seq_starts += num_decode, state_slots += num_decode;
+        num_seqs -= num_decode;
+        if (num_seqs == 0) {
+            hipLaunchKernelGGL((retention_finish_kernel<elem_t>), dim3((unsigned)tokens, (unsigned)heads), dim3(NVA_WAVE), 0,
+                               stream, o_raw, (int64_t)heads * vdim, gate, stride, (elem_t*)y, y_stride, vdim, eps);
+            return nva_check_launch("retention_finish");
+        }
+    }
     if (matrix_cores && dim % 32 == 0 && dim <= 256 && vdim % 32 == 0) {
         // positions: int32 [tokens]; cos_sin: float [tokens, rot] scratch (both needed with a rotation)
         if (rot && (!positions || !cos_sin)) return nva_fail("retention: the rotation needs positions and room for the angles");
@@ -360,23 +545,29 @@ NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* 
                                inv_freq, rot / 2, cos_sin, total);
         }
         const int nsl = vdim / 32;
-        const int waves = nsl < RET_MFMA_WAVES ? nsl : RET_MFMA_WAVES;
+        const int waves = nsl <= 2 ? nsl : RET_MFMA_WAVES;
+        // loads of eight elements: rows and parts of rows that start at multiples of eight elements, 16 bytes
+        // aligned, and a rotation whose halves are multiples of eight channels
+        const int vec = stride % 8 == 0 && nva_aligned(proj, 8 * sizeof(elem_t) > 16 ? 16 : 8 * sizeof(elem_t)) &&
+                        rot % 16 == 0 && (!rot || nva_aligned(cos_sin, 16));
         const int groups = (nsl + waves - 1) / waves;
         const size_t bytes = ret_mfma_lds_floats(dim, waves) * sizeof(float);
         dim3 grid((unsigned)(heads * groups), (unsigned)num_seqs);
-#define RET_LAUNCH(DTT)                                                                                             \
+#define RET_LAUNCH_W(DTT, NWW)                                                                                      \
         {                                                                                                           \
-            auto kernel = retention_mfma_kernel<elem_t, DTT>;                                                        \
+            auto kernel = retention_mfma_kernel<elem_t, DTT, NWW>;                                                   \
             static bool raised = false;                                                                              \
             if (!raised && bytes > 48 * 1024) {                                                                       \
                 if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) \
                     return nva_fail("retention: cannot have %zu bytes of LDS", bytes);                               \
                 raised = true;                                                                                       \
             }                                                                                                        \
-            hipLaunchKernelGGL(kernel, grid, dim3(waves * NVA_WAVE), bytes, stream, p, stride, o_raw,               \
+            hipLaunchKernelGGL(kernel, grid, dim3(NWW * NVA_WAVE), bytes, stream, p, stride, o_raw,                 \
                                (int64_t)heads * vdim, state, cu_seqlens_q, seq_starts, state_slots, decay_pow, cos_sin, \
-                               rot, heads, vdim, k_scale);                                                           \
+                               rot, heads, vdim, k_scale, vec);                                                      \
         }
+#define RET_LAUNCH(DTT)                                                                                             \
+        if (waves == 1) RET_LAUNCH_W(DTT, 1) else if (waves == 2) RET_LAUNCH_W(DTT, 2) else RET_LAUNCH_W(DTT, 4)
         switch (dim / 32) {
             case 1: RET_LAUNCH(1); break;
             case 2: RET_LAUNCH(2); break;
@@ -387,10 +578,10 @@ NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* 
             case 7: RET_LAUNCH(7); break;
             default: RET_LAUNCH(8); break;
         }
+#undef RET_LAUNCH_W
 #undef RET_LAUNCH
         int rc = nva_check_launch("retention (matrix cores)");
         if (rc) return rc;
-        const elem_t* gate = p + (int64_t)2 * heads * dim + (int64_t)heads * vdim;
         hipLaunchKernelGGL((retention_finish_kernel<elem_t>), dim3((unsigned)tokens, (unsigned)heads), dim3(NVA_WAVE), 0,
                            stream, o_raw, (int64_t)heads * vdim, gate, stride, (elem_t*)y, y_stride, vdim, eps);
         return nva_check_launch("retention_finish");
@@ -411,7 +602,6 @@ NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* 
                        inv_freq, rot, heads, dim, vdim, vslice, nslices, k_scale);
     int rc = nva_check_launch("retention");
     if (rc) return rc;
-    const elem_t* gate = p + (int64_t)2 * heads * dim + (int64_t)heads * vdim;
     hipLaunchKernelGGL((retention_finish_kernel<elem_t>), dim3((unsigned)tokens, (unsigned)heads), dim3(NVA_WAVE), 0, stream,
                        o_raw, (int64_t)heads * vdim, gate, stride, (elem_t*)y, y_stride, vdim, eps);
     return nva_check_launch("retention_finish");

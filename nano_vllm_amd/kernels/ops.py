@@ -254,6 +254,8 @@ class HipKernels:
         self.mfma_attention = True
         # False: retention always runs the general kernel
         self.mfma_retention = True
+        # False: single tokens run the chunked kernels as chunks of one token
+        self.retention_decode_kernel = True
         # False: the general kernel runs one wave per token for portions of prompts too (the same bits, slower)
         self.tiled_general_attention = True
 
@@ -1038,8 +1040,8 @@ class HipKernels:
         _i32(batch.cu_seqlens_q, seqs + 1, "cu_seqlens_q")
         _i32(batch.seq_starts, seqs, "seq_starts")
         _i32(batch.state_slots, seqs, "state_slots")
-        if sum(batch.q_lens) != tokens:
-            raise KernelError("retention: the batch does not describe the projections' rows")
+        if sum(batch.q_lens) != tokens or any(n != 1 for n in batch.q_lens[:batch.num_decode]):
+            raise KernelError("retention: the batch does not describe the projections' rows (single tokens first)")
         if out is None:
             out = torch.empty((tokens, heads * v_dim), dtype=proj.dtype, device=proj.device)
         orows, ow, os_ = _rows2d(out, "retention output")
@@ -1060,7 +1062,8 @@ class HipKernels:
                      _p(state), c_i64(state.shape[0]), _p(batch.cu_seqlens_q), _p(batch.seq_starts),
                      _p(batch.state_slots), c_i64(seqs), c_i64(tokens), _p(decay_powers), _p(inv_freq), c_i32(rot),
                      c_i32(heads), c_i32(dim), c_i32(v_dim), c_i32(vslice), c_f32(k_scale), c_f32(eps), _p(positions),
-                     _p(scratch), c_i32(1 if self.mfma_retention else 0), self._stream())
+                     _p(scratch), c_i32(1 if self.mfma_retention else 0),
+                     c_i64(batch.num_decode if self.retention_decode_kernel else 0), self._stream())
         return out
 
     @staticmethod

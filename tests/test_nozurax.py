@@ -300,6 +300,7 @@ def _plain_retention_of_projections(proj, heads, dim, vdim, decay, rot, base, ep
 def _state_batch(dev, q_lens, starts, slots):
     return SimpleNamespace(
         num_seqs=len(q_lens), q_lens=list(q_lens), starts=list(starts),
+        num_decode=next((i for i, n in enumerate(q_lens) if n != 1), len(q_lens)),
         positions=torch.tensor([p for s, n in zip(starts, q_lens) for p in range(s, s + n)], dtype=torch.int32, device=dev),
         cu_seqlens_q=torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32, device=dev),
         seq_starts=torch.tensor(starts, dtype=torch.int32, device=dev),
