@@ -255,6 +255,13 @@ __host__ __device__ inline size_t ret_mfma_lds_floats(int dim, int waves) {
     return (size_t)2 * RET_C * (dim + 1) + (size_t)waves * 2 * RET_C * (RET_C + 1) + 64;
 }
 
+// A long portion is cut into blocks of `bt` tokens (units: int32 [n][4] = request, first token of the
+// block within the portion, its tokens, blocks of the portion) that run side by side, each from a
+// zero state but the first: mode 0 leaves a block's outputs without what the state at its start
+// would give, and the block's own end state in scratch[unit] (a portion of one block writes the
+// request's slot itself); retention_scan_kernel then makes every block's true end state,
+// E_b = decay^len_b E_(b-1) + (end state from zero), and the request's new state; mode 1 adds
+// decay^(i+1) q_i E_(b-1) to the outputs of every block but the first.  units null: one block a request.
 // NW: waves of the workgroup.  vec: rows, offsets and the rotation allow loads of eight elements; the
 // chunk after the one at hand is then asked for before the products start and waits in registers.
 template <typename T, int DT, int NW>
@@ -263,7 +270,8 @@ retention_mfma_kernel(const T* __restrict__ proj, int64_t stride, float* __restr
                       float* __restrict__ state, const int32_t* __restrict__ cu_seqlens_q,
                       const int32_t* __restrict__ seq_starts, const int32_t* __restrict__ state_slots,
                       const float* __restrict__ decay_pow, const float* __restrict__ cos_sin, int rot,
-                      int heads, int vdim, float k_scale, int vec) {
+                      int heads, int vdim, float k_scale, int vec, const int32_t* __restrict__ units,
+                      float* __restrict__ scratch, int mode) {
     static_assert(RET_C == 32, "a chunk is one MFMA tile of rows");
     constexpr int D = 32 * DT, DS = D + 1, VS = RET_C + 1;
     extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -281,12 +289,21 @@ retention_mfma_kernel(const T* __restrict__ proj, int64_t stride, float* __restr
     const int slice = (blockIdx.x % groups) * waves + wave;
     const bool active = slice < nslices;                      // a wave without a slice only helps to load q and k
     const int c0 = 32 * (active ? slice : 0);
-    const int seq = blockIdx.y;
-    const int q_begin = cu_seqlens_q[seq];
-    const int q_len = cu_seqlens_q[seq + 1] - q_begin;
-    const int start = seq_starts[seq];
+    int seq = blockIdx.y, first_token = 0, unit_len = -1, blocks = 1;
+    if (units) {
+        const int32_t* u = units + 4 * (int64_t)blockIdx.y;
+        seq = u[0], first_token = u[1], unit_len = u[2], blocks = u[3];
+    }
+    if (mode == 1 && first_token == 0) return;                  // a first block has its state from the start
+    const int q_begin = cu_seqlens_q[seq] + first_token;
+    const int q_len = units ? unit_len : cu_seqlens_q[seq + 1] - q_begin;
+    // a block after the first starts from zero (mode 0) or reads the block before's end state (mode 1)
+    const int start = first_token == 0 ? seq_starts[seq] : 0;
     const int slot = state_slots[seq];
-    float* const s_g = state + (((int64_t)slot * heads + h) * D) * vdim + c0 + col;
+    float* const s_slot = state + (((int64_t)slot * heads + h) * D) * vdim + c0 + col;
+    float* const s_unit = scratch ? scratch + (((int64_t)blockIdx.y * heads + h) * D) * vdim + c0 + col : s_slot;
+    const float* const s_from = mode == 1 ? s_unit - (int64_t)heads * D * vdim : s_slot;
+    float* const s_to = blocks == 1 ? s_slot : s_unit;
     const int half = rot / 2;
     const int64_t q_off = (int64_t)h * D, k_off = (int64_t)(heads + h) * D;
     const int64_t v_off = (int64_t)2 * heads * D + (int64_t)h * vdim + c0;
@@ -298,7 +315,9 @@ retention_mfma_kernel(const T* __restrict__ proj, int64_t stride, float* __restr
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) S[dt][r] = start > 0 && active ? s_g[(int64_t)(32 * dt + rowmap(r)) * vdim] : 0.f;
+        for (int r = 0; r < 16; ++r)
+            S[dt][r] = (start > 0 || mode == 1) && active ? s_from[(int64_t)(32 * dt + rowmap(r)) * vdim] : 0.f;
+    float chunks_decay = 1.f;                     // decay^(32 c) at the block's chunk c (mode 1)
 
     // blocks of eight elements: of q and k [32][D / 8] over all threads, of v [32][4] over a wave's lanes
     constexpr int QK_BLOCKS = RET_C * D / 8, PQ = (QK_BLOCKS + NW * NVA_WAVE - 1) / (NW * NVA_WAVE);
@@ -404,8 +423,31 @@ retention_mfma_kernel(const T* __restrict__ proj, int64_t stride, float* __restr
         }
         }
         __syncthreads();
-        // ---- scores: A[i][j] = q_i . k_j
         f32x16 acc;
+        if (mode == 1) {
+            // ---- what the state at the block's start gives, added to the outputs that are there
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = rowmap(r);
+                acc[r] = i < n && active ? o_raw[(int64_t)(q_begin + t0 + i) * o_stride + (int64_t)h * vdim + c0 + col] : 0.f;
+            }
+            const float row_decay = pw_s[col + 1] * chunks_decay;
+            const float* qa = q_s + col * DS + 4 * up;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[32 * dt + 8 * (r >> 2) + (r & 3)] * row_decay, S[dt][r],
+                                                               acc, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = rowmap(r);
+                if (i < n && active) o_raw[(int64_t)(q_begin + t0 + i) * o_stride + (int64_t)h * vdim + c0 + col] = acc[r];
+            }
+            chunks_decay *= pw_s[RET_C];
+            continue;
+        }
+        // ---- scores: A[i][j] = q_i . k_j
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
         {
@@ -465,11 +507,35 @@ retention_mfma_kernel(const T* __restrict__ proj, int64_t stride, float* __restr
             }
         }
     }
-    if (!active) return;
+    if (!active || mode == 1) return;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s_g[(int64_t)(32 * dt + rowmap(r)) * vdim] = S[dt][r];
+        for (int r = 0; r < 16; ++r) s_to[(int64_t)(32 * dt + rowmap(r)) * vdim] = S[dt][r];
+}
+
+// The blocks' end states from zero, one after the other, into their true end states, and the last
+// into the request's slot.  chains: int32 [n][4] = first unit, blocks, request, tokens of the last block.
+__global__ void __launch_bounds__(256)
+retention_scan_kernel(float* __restrict__ scratch, float* __restrict__ state, const int32_t* __restrict__ chains,
+                      const int32_t* __restrict__ state_slots, const float* __restrict__ decay_pow, int heads,
+                      int64_t per_head, int bt) {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= heads * per_head) return;
+    const int32_t* c = chains + 4 * (int64_t)blockIdx.y;
+    const int first_unit = c[0], blocks = c[1], seq = c[2], last_len = c[3];
+    const float* pw = decay_pow + (e / per_head) * (RET_C + 1);
+    float whole = 1.f, last = pw[last_len % RET_C];
+    for (int i = 0; i < bt / RET_C; ++i) whole *= pw[RET_C];
+    for (int i = 0; i < last_len / RET_C; ++i) last *= pw[RET_C];
+    const int64_t unit = heads * per_head;
+    float* at = scratch + (int64_t)first_unit * unit + e;
+    float E = at[0];
+    for (int b = 1; b < blocks; ++b) {
+        E = (b == blocks - 1 ? last : whole) * E + at[b * unit];
+        at[b * unit] = E;
+    }
+    state[(int64_t)state_slots[seq] * unit + e] = E;
 }
 
 // y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * silu(g[t, h, :]); one wave per (token, head).
@@ -504,7 +570,8 @@ NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* 
                                        int64_t tokens, const float* decay_pow, const float* inv_freq, int rot,
                                        int heads, int dim, int vdim, int vslice, float k_scale, float eps,
                                        const int32_t* positions, float* cos_sin, int matrix_cores, int64_t num_decode,
-                                       hipStream_t stream) {
+                                       const int32_t* units, int64_t num_units, const int32_t* chains,
+                                       int64_t num_chains, int block_tokens, float* block_states, hipStream_t stream) {
     if (num_seqs == 0 || tokens == 0) return 0;
     if (num_seqs < 0 || num_seqs > 65535 || tokens < 0 || tokens > 0x7fffffff)
         return nva_fail("retention: bad counts requests=%lld tokens=%lld", (long long)num_seqs, (long long)tokens);
@@ -552,7 +619,20 @@ NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* 
                         rot % 16 == 0 && (!rot || nva_aligned(cos_sin, 16));
         const int groups = (nsl + waves - 1) / waves;
         const size_t bytes = ret_mfma_lds_floats(dim, waves) * sizeof(float);
-        dim3 grid((unsigned)(heads * groups), (unsigned)num_seqs);
+        // units: the portions cut into blocks that run side by side (see retention_mfma_kernel); the requests
+        // they name are counted from the first that brings a portion
+        if (units && (num_units <= 0 || num_units > 65535 || !block_states || block_tokens < RET_C || block_tokens % RET_C ||
+                      num_chains < 0 || num_chains > 65535 || (num_chains && !chains)))
+            return nva_fail("retention: bad blocks (%lld units, %lld chains, %d tokens a block)", (long long)num_units,
+                            (long long)num_chains, block_tokens);
+        dim3 grid((unsigned)(heads * groups), (unsigned)(units ? num_units : num_seqs));
+        for (int mode = 0; mode < (units && num_chains ? 2 : 1); ++mode) {
+        if (mode == 1) {
+            const int64_t per_head = (int64_t)dim * vdim;
+            hipLaunchKernelGGL(retention_scan_kernel, dim3((unsigned)((heads * per_head + 255) / 256), (unsigned)num_chains),
+                               dim3(256), 0, stream, block_states, state, chains, state_slots, decay_pow, heads, per_head,
+                               block_tokens);
+        }
 #define RET_LAUNCH_W(DTT, NWW)                                                                                      \
         {                                                                                                           \
             auto kernel = retention_mfma_kernel<elem_t, DTT, NWW>;                                                   \
@@ -564,7 +644,7 @@ NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* 
             }                                                                                                        \
             hipLaunchKernelGGL(kernel, grid, dim3(NWW * NVA_WAVE), bytes, stream, p, stride, o_raw,                 \
                                (int64_t)heads * vdim, state, cu_seqlens_q, seq_starts, state_slots, decay_pow, cos_sin, \
-                               rot, heads, vdim, k_scale, vec);                                                      \
+                               rot, heads, vdim, k_scale, vec, units, units ? block_states : nullptr, mode);         \
         }
 #define RET_LAUNCH(DTT)                                                                                             \
         if (waves == 1) RET_LAUNCH_W(DTT, 1) else if (waves == 2) RET_LAUNCH_W(DTT, 2) else RET_LAUNCH_W(DTT, 4)
@@ -580,6 +660,7 @@ NVA_EXPORT int NVA_NAME(nva_retention)(const void* proj, int64_t stride, float* 
         }
 #undef RET_LAUNCH_W
 #undef RET_LAUNCH
+        }
         int rc = nva_check_launch("retention (matrix cores)");
         if (rc) return rc;
         hipLaunchKernelGGL((retention_finish_kernel<elem_t>), dim3((unsigned)tokens, (unsigned)heads), dim3(NVA_WAVE), 0,

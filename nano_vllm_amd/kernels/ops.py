@@ -128,6 +128,28 @@ PREFILL_MAX_TABLE = 4096    # pages of a block-table row the prefill attention k
 GENERAL_TILED_MAX_HEAD_DIM = 128    # head sizes of nva_paged_attention_tiled
 
 
+def retention_blocks(q_lens, first_seq: int):
+    """How the retention kernel on the matrix cores cuts the step's portions (the requests from
+    `first_seq` on) into blocks that run side by side: (tokens of a block, units, chains) with units a
+    flat list of (request counted from first_seq, first token of the block within the portion, its
+    tokens, blocks of the portion) and chains one of (first unit, blocks, request, tokens of the last
+    block) for every portion of more than one block.  Blocks of 64 tokens, of more where that still
+    leaves 64 blocks."""
+    total = sum(q_lens[first_seq:])
+    bt = 64
+    while bt < 512 and total // bt > 64:
+        bt *= 2
+    units, chains = [], []
+    for s in range(first_seq, len(q_lens)):
+        n = q_lens[s]
+        nb = (n + bt - 1) // bt
+        if nb > 1:
+            chains += [len(units) // 4, nb, s - first_seq, n - (nb - 1) * bt]
+        for b in range(nb):
+            units += [s - first_seq, b * bt, min(bt, n - b * bt), nb]
+    return bt, units, chains
+
+
 def prefill_tile_order(q_lens, starts, first_seq: int) -> list:
     """Flat [(request, row tile), ...] of the requests from `first_seq` on, from the tile that
     sees the most keys to the one that sees the fewest: the prefill attention kernel hands its
@@ -256,6 +278,8 @@ class HipKernels:
         self.mfma_retention = True
         # False: single tokens run the chunked kernels as chunks of one token
         self.retention_decode_kernel = True
+        # False: a portion's chunks always run one after the other
+        self.retention_blocks_side_by_side = True
         # False: the general kernel runs one wave per token for portions of prompts too (the same bits, slower)
         self.tiled_general_attention = True
 
@@ -1058,12 +1082,33 @@ class HipKernels:
             _i32(batch.positions, tokens, "positions")
             positions = batch.positions
             scratch = torch.empty((tokens, rot), dtype=torch.float32, device=proj.device)
+        # long portions are cut into blocks that run side by side (the same cut for every layer of the step)
+        units = chains = block_states = None
+        bt = n_units = n_chains = 0
+        first = batch.num_decode if self.retention_decode_kernel else 0
+        if self.mfma_retention and dim % 32 == 0 and dim <= 256 and v_dim % 32 == 0 and self.retention_blocks_side_by_side:
+            kept = getattr(batch, "step_cache", None)
+            if kept is None:
+                kept = batch.step_cache = {}
+            plan = kept.get(("retention_blocks", first))
+            if plan is None:
+                bt, flat_units, flat_chains = retention_blocks(batch.q_lens, first)
+                if flat_chains:
+                    both = torch.tensor(flat_units + flat_chains, dtype=torch.int32).to(proj.device, non_blocking=True)
+                    plan = (bt, len(flat_units) // 4, len(flat_chains) // 4, both[: len(flat_units)], both[len(flat_units):])
+                else:
+                    plan = (0, 0, 0, None, None)
+                kept[("retention_blocks", first)] = plan
+            bt, n_units, n_chains, units, chains = plan
+            if n_chains:
+                block_states = torch.empty((n_units, heads, dim, v_dim), dtype=torch.float32, device=proj.device)
         library.call("retention", _suffix(proj), "nva_retention", _p(proj), c_i64(stride), _p(raw), _p(out), c_i64(os_),
                      _p(state), c_i64(state.shape[0]), _p(batch.cu_seqlens_q), _p(batch.seq_starts),
                      _p(batch.state_slots), c_i64(seqs), c_i64(tokens), _p(decay_powers), _p(inv_freq), c_i32(rot),
                      c_i32(heads), c_i32(dim), c_i32(v_dim), c_i32(vslice), c_f32(k_scale), c_f32(eps), _p(positions),
                      _p(scratch), c_i32(1 if self.mfma_retention else 0),
-                     c_i64(batch.num_decode if self.retention_decode_kernel else 0), self._stream())
+                     c_i64(first), _p(units), c_i64(n_units), _p(chains), c_i64(n_chains), c_i32(bt), _p(block_states),
+                     self._stream())
         return out
 
     @staticmethod

@@ -384,6 +384,42 @@ def test_retention_of_unequal_requests_in_one_batch(backend):
     assert bool(torch.isnan(state[2]).all())                         # the slot that no request holds
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_retention_of_long_portions_whose_blocks_run_side_by_side(dtype):
+    # portions of many blocks beside a short one and one that continues a state; with the blocks one
+    # after the other the same numbers but for rounding
+    k, dev = _kernels("hip", dtype)
+    heads, dim, vdim, decay, rot, base = 2, 64, 96, (0.9, 0.9995), 32, 1e4
+    powers, inv_freq = _retention_constants(k, dev, decay, dim, rot, base)
+    lens = [700, 40, 333]
+    first = [0, 0, 100]                       # request 2 has 100 tokens in its state already
+    projs = [_retention_inputs(heads, dim, vdim, n, 30 + i, dtype) for i, n in enumerate(lens)]
+    wants = [_plain_retention_of_projections(p, heads, dim, vdim, decay, rot, base, 1e-6) for p in projs]
+    results = {}
+    for side_by_side in (True, False):
+        k.retention_blocks_side_by_side = side_by_side
+        try:
+            state = torch.full((3, heads, dim, vdim), float("nan"), dtype=torch.float32, device=dev)
+            k.retention(projs[2][:100].contiguous().to(dev), heads, dim, vdim, state, powers, inv_freq, dim ** -0.5, 1e-6,
+                        _state_batch(dev, [100], [0], [2]))
+            x = torch.cat([p[f:] for p, f in zip(projs, first)]).to(dev)
+            batch = _state_batch(dev, [n - f for n, f in zip(lens, first)], first, [0, 1, 2])
+            got = k.retention(x, heads, dim, vdim, state, powers, inv_freq, dim ** -0.5, 1e-6, batch).float().cpu()
+            results[side_by_side] = (got, state.clone())
+        finally:
+            k.retention_blocks_side_by_side = True
+        at = 0
+        for want, f in zip(wants, first):
+            n = want.shape[0] - f
+            e = float((got[at:at + n].double() - want[f:]).abs().max() / want.abs().max())
+            assert e < (3e-5 if dtype == torch.float32 else 2e-2), (side_by_side, e)
+            at += n
+    assert float((results[True][0] - results[False][0]).abs().max()) < (1e-4 if dtype == torch.float32 else 5e-2)
+    a, b = results[True][1], results[False][1]
+    assert float((a - b).abs().max() / b.abs().max()) < 1e-5          # the states the requests are left with
+
+
 @pytest.mark.parametrize("backend", BACKENDS)
 def test_retention_keeps_a_far_token_by_its_decay(backend):
     # token 0 carries a large key and value; a query like its key stands 400 tokens later: the head
