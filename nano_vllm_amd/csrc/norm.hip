@@ -180,11 +180,14 @@ NVA_EXPORT int NVA_NAME(nva_rms_norm_of_partials)(const float* sums, int splits,
 //     r <- r + a + b        (else; a and b may each be absent)
 //     y = r * rsqrt(mean(r^2) + eps) * (offset + w)        rounded once, to the element type
 // All arithmetic in float.  offset 1 is the weight stored around zero, offset 0 the plain weight.
+// An addend may be given as the float partial sums of a product whose k range was split (pa, pb): they
+// are added, with the bias, and rounded to the element type as the product's own finishing pass would.
 template <typename T>
 __global__ void __launch_bounds__(512)
-stream_rms_norm_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ b, int64_t b_stride,
-                       float* residual, int64_t r_stride, int first, const void* __restrict__ weight, int w_is_f32,
-                       float offset, T* __restrict__ y, int64_t y_stride, int width, float eps) {
+stream_rms_norm_kernel(const T* __restrict__ a, int64_t a_stride, PartialInput pa, const T* __restrict__ b,
+                       int64_t b_stride, PartialInput pb, float* residual, int64_t r_stride, int first,
+                       const void* __restrict__ weight, int w_is_f32, float offset, T* __restrict__ y,
+                       int64_t y_stride, int width, float eps) {
     __shared__ float scratch[16];
     const int64_t row = blockIdx.x;
     const T* ar = a ? a + row * a_stride : nullptr;
@@ -201,10 +204,10 @@ stream_rms_norm_kernel(const T* __restrict__ a, int64_t a_stride, const T* __res
         float s = first ? 0.f : rr[i];
         // the two sublayers are added to each other first, then to the stream
         float add = 0.f;
-        if (ar) add = to_float(ar[i]);
-        if (br) add += to_float(br[i]);
+        if (pa.sums) add = partial_value<T>(pa, row, width, i); else if (ar) add = to_float(ar[i]);
+        if (pb.sums) add += partial_value<T>(pb, row, width, i); else if (br) add += to_float(br[i]);
         s += add;
-        if (ar || br || first) rr[i] = s;
+        if (ar || br || pa.sums || pb.sums || first) rr[i] = s;
         if (n < KEEP) kept[n] = s;
         ss += s * s;
     }
@@ -219,7 +222,11 @@ stream_rms_norm_kernel(const T* __restrict__ a, int64_t a_stride, const T* __res
 }
 
 // residual: float [rows, width] in place.  a, b: elements or null.  first != 0: the stream starts with a (+ b).
-NVA_EXPORT int NVA_NAME(nva_stream_rms_norm)(const void* a, int64_t a_stride, const void* b, int64_t b_stride,
+// a_sums / b_sums (with splits, the stride between splits and an optional bias): the addend as partial sums
+// [splits][rows][width] instead of elements.
+NVA_EXPORT int NVA_NAME(nva_stream_rms_norm)(const void* a, int64_t a_stride, const float* a_sums, int a_splits,
+                                             int64_t a_split_stride, const void* a_bias, const void* b, int64_t b_stride,
+                                             const float* b_sums, int b_splits, int64_t b_split_stride, const void* b_bias,
                                              float* residual, int64_t r_stride, int first, const void* weight,
                                              int w_is_f32, float offset, void* y, int64_t y_stride, int64_t rows,
                                              int width, float eps, hipStream_t stream) {
@@ -227,10 +234,14 @@ NVA_EXPORT int NVA_NAME(nva_stream_rms_norm)(const void* a, int64_t a_stride, co
     if (rows < 0 || rows > 0x7fffffff || width <= 0)
         return nva_fail("stream_rms_norm: bad shape rows=%lld width=%d", (long long)rows, width);
     if (!residual || !y || !weight) return nva_fail("stream_rms_norm: residual, output and weight are needed");
-    if (first && !a) return nva_fail("stream_rms_norm: the stream starts with an addend");
+    if (first && !a && !a_sums) return nva_fail("stream_rms_norm: the stream starts with an addend");
+    const PartialInput pa{a_sums, a_splits, a_split_stride, a_bias}, pb{b_sums, b_splits, b_split_stride, b_bias};
+    if ((a_sums && (a_splits <= 0 || a_split_stride < rows * (int64_t)width)) ||
+        (b_sums && (b_splits <= 0 || b_split_stride < rows * (int64_t)width)))
+        return nva_fail("stream_rms_norm: bad partial sums");
     const int threads = width >= 2048 ? 512 : width >= 1024 ? 256 : width >= 256 ? 128 : 64;
     hipLaunchKernelGGL((stream_rms_norm_kernel<elem_t>), dim3((unsigned)rows), dim3(threads), 0, stream,
-                       (const elem_t*)a, a_stride, (const elem_t*)b, b_stride, residual, r_stride, first, weight,
+                       (const elem_t*)a, a_stride, pa, (const elem_t*)b, b_stride, pb, residual, r_stride, first, weight,
                        w_is_f32, offset, (elem_t*)y, y_stride, width, eps);
     return nva_check_launch("stream_rms_norm");
 }

@@ -8,8 +8,9 @@
 //     cache <- k, v                                        at the token's slot (slot < 0: nothing is written)
 //
 // The row is the packed projection [q | k | v] of Hq * D, Hkv * D and Hkv * DV entries, biases added
-// by the product.  Sums of squares, scales, the logarithm and the products are float; q is written
-// back in place and k, v into the cache, each rounded once to the element type.  The weights are
+// by the product (or still to be added: the row may come as the float partial sums of a product whose
+// k range was split, which are added up here).  Sums of squares, scales, the logarithm and the products
+// are float; q is written out and k, v into the cache, each rounded once to the element type.  The weights are
 // plain (not one-plus), stored as elements or float.
 // Cache layout: K [pages, Hkv, page, D], V [pages, Hkv, page / vt, DV, vt] (common.h).
 // One workgroup per token.
@@ -17,67 +18,65 @@
 
 template <typename T>
 __global__ void __launch_bounds__(256)
-qk_rownorm_store_kernel(T* __restrict__ qkv, int64_t stride, int num_heads, int num_kv_heads, int head_dim, int v_dim,
+qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput part, T* __restrict__ q_out,
+                        int64_t q_stride, int num_heads, int num_kv_heads, int head_dim, int v_dim,
                         const void* __restrict__ q_weight, const void* __restrict__ k_weight, int w_is_f32, float eps,
                         const int32_t* __restrict__ positions, float temp_coef, int temp_every,
                         const int32_t* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
                         int page_size) {
+    extern __shared__ __attribute__((aligned(16))) float row_s[];      // the token's row, as float
     __shared__ float scratch[16];
     const int64_t t = blockIdx.x;
-    T* row = qkv + t * stride;
     const int qd = num_heads * head_dim, kd = num_kv_heads * head_dim, vd = num_kv_heads * v_dim;
+    const int width = qd + kd + vd;
     const int tid = threadIdx.x;
+    // what the slot and the position say is asked for before the row arrives
+    const int slot = slots ? slots[t] : -1;
+    const int steps = temp_coef != 0.f ? (positions[t] + 1) / temp_every : 0;
 
     float sq = 0.f, sk = 0.f;
-    for (int i = tid; i < qd; i += blockDim.x) {
-        const float x = to_float(row[i]);
-        sq += x * x;
-    }
-    for (int i = tid; i < kd; i += blockDim.x) {
-        const float x = to_float(row[qd + i]);
-        sk += x * x;
+    for (int i = tid; i < width; i += blockDim.x) {
+        const float x = part.sums ? partial_value<T>(part, t, width, i) : to_float(qkv[t * stride + i]);
+        row_s[i] = x;
+        if (i < qd) sq += x * x; else if (i < qd + kd) sk += x * x;
     }
     sq = block_sum(sq, scratch);
     sk = kd ? block_sum(sk, scratch) : 0.f;
 
     float q_scale = q_weight ? rsqrtf(sq / (float)qd + eps) : 1.f;
-    if (temp_coef != 0.f) {
-        const int steps = (positions[t] + 1) / temp_every;
-        q_scale *= 1.f + temp_coef * logf((float)steps + 1.f);
-    }
+    if (temp_coef != 0.f) q_scale *= 1.f + temp_coef * logf((float)steps + 1.f);
+    T* qrow = q_out + t * q_stride;
     for (int i = tid; i < qd; i += blockDim.x) {
         const float w = !q_weight ? 1.f : w_is_f32 ? static_cast<const float*>(q_weight)[i]
                                                    : to_float(static_cast<const T*>(q_weight)[i]);
-        row[i] = from_float<T>(to_float(row[i]) * q_scale * w);
+        qrow[i] = from_float<T>(row_s[i] * q_scale * w);
     }
-    if (!kd) return;
-    const int slot = slots ? slots[t] : -1;
+    if (!kd || slot < 0 || !k_cache) return;
     const float k_scale = k_weight ? rsqrtf(sk / (float)kd + eps) : 1.f;
-    const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+    const int page = slot / page_size, off = slot % page_size;
     const int vt = nva_v_tile(page_size);
     for (int i = tid; i < kd; i += blockDim.x) {
         const float w = !k_weight ? 1.f : w_is_f32 ? static_cast<const float*>(k_weight)[i]
                                                    : to_float(static_cast<const T*>(k_weight)[i]);
-        const T k = from_float<T>(to_float(row[qd + i]) * k_scale * w);
-        row[qd + i] = k;
-        if (slot >= 0 && k_cache) {
-            const int g = i / head_dim, d = i % head_dim;
-            k_cache[(((int64_t)page * num_kv_heads + g) * page_size + off) * head_dim + d] = k;
-        }
+        const int g = i / head_dim, d = i % head_dim;
+        k_cache[(((int64_t)page * num_kv_heads + g) * page_size + off) * head_dim + d] =
+            from_float<T>(row_s[qd + i] * k_scale * w);
     }
-    if (slot >= 0 && v_cache) {
-        for (int i = tid; i < vd; i += blockDim.x) {
-            const int g = i / v_dim, d = i % v_dim;
-            v_cache[((int64_t)page * num_kv_heads + g) * v_dim * (int64_t)page_size + nva_v_offset(off, d, v_dim, vt)] =
-                row[qd + kd + i];
-        }
+    for (int i = tid; i < vd; i += blockDim.x) {
+        const int g = i / v_dim, d = i % v_dim;
+        v_cache[((int64_t)page * num_kv_heads + g) * v_dim * (int64_t)page_size + nva_v_offset(off, d, v_dim, vt)] =
+            from_float<T>(row_s[qd + kd + i]);
     }
 }
 
-// qkv: [tokens, Hq * D + Hkv * D + Hkv * DV] with rows `stride` elements apart, q and k rewritten in place.
+// qkv: [tokens, Hq * D + Hkv * D + Hkv * DV] with rows `stride` elements apart, or (sums != null) the float
+// partial sums [splits][tokens][width] of the projection with its bias, which are added up here.
+// q_out: [tokens, Hq * D] with rows q_stride apart (it may be qkv itself: q is then rewritten in place).
 // q_weight [Hq * D], k_weight [Hkv * D]: both or none.  positions are needed with a temperature.
 // slots (with the caches) may be null: nothing is stored then.  num_kv_heads 0: the row holds q only.
-NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(void* qkv, int64_t stride, int64_t tokens, int num_heads, int num_kv_heads,
+NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(const void* qkv, int64_t stride, const float* sums, int splits,
+                                              int64_t split_stride, const void* bias, void* q_out, int64_t q_stride,
+                                              int64_t tokens, int num_heads, int num_kv_heads,
                                               int head_dim, int v_dim, const void* q_weight, const void* k_weight,
                                               int w_is_f32, float eps, const int32_t* positions, float temp_coef,
                                               int temp_every, const int32_t* slots, void* k_cache, void* v_cache,
@@ -88,16 +87,29 @@ NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(void* qkv, int64_t stride, int64_t
         return nva_fail("qk_rownorm_store: bad sizes heads=%d kv_heads=%d head_dim=%d v_dim=%d", num_heads, num_kv_heads,
                         head_dim, v_dim);
     const int64_t width = (int64_t)(num_heads + num_kv_heads) * head_dim + (int64_t)num_kv_heads * v_dim;
-    if (stride < width) return nva_fail("qk_rownorm_store: rows of %lld elements are %lld apart", (long long)width, (long long)stride);
+    if (width > 36 * 1024) return nva_fail("qk_rownorm_store: a row of %lld entries does not fit the LDS", (long long)width);
+    if (!sums && (!qkv || stride < width))
+        return nva_fail("qk_rownorm_store: rows of %lld elements are %lld apart", (long long)width, (long long)stride);
+    if (sums && (splits <= 0 || split_stride < tokens * width)) return nva_fail("qk_rownorm_store: bad partial sums");
+    if (!q_out || q_stride < (int64_t)num_heads * head_dim) return nva_fail("qk_rownorm_store: no room for q");
     if (num_kv_heads && (q_weight == nullptr) != (k_weight == nullptr))
         return nva_fail("qk_rownorm_store: give both norm weights or none");
     if (temp_coef != 0.f && (!positions || temp_every <= 0))
         return nva_fail("qk_rownorm_store: a query temperature needs positions and a positive step");
     if ((k_cache || v_cache) && (!k_cache || !v_cache || !slots || page_size <= 0 || !num_kv_heads))
         return nva_fail("qk_rownorm_store: storing needs both caches, the slots and the page size");
-    hipLaunchKernelGGL((qk_rownorm_store_kernel<elem_t>), dim3((unsigned)tokens), dim3(256), 0, stream, (elem_t*)qkv,
-                       stride, num_heads, num_kv_heads, head_dim, v_dim, q_weight, k_weight, w_is_f32, eps, positions,
-                       temp_coef, temp_every, slots, (elem_t*)k_cache, (elem_t*)v_cache, page_size);
+    auto kernel = qk_rownorm_store_kernel<elem_t>;
+    const size_t lds = (size_t)width * sizeof(float);
+    static bool raised = false;
+    if (!raised && lds > 48 * 1024) {
+        if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+            return nva_fail("qk_rownorm_store: cannot have %zu bytes of LDS", lds);
+        raised = true;
+    }
+    const PartialInput part{sums, splits, split_stride, bias};
+    hipLaunchKernelGGL(kernel, dim3((unsigned)tokens), dim3(256), lds, stream, (const elem_t*)qkv, stride, part,
+                       (elem_t*)q_out, q_stride, num_heads, num_kv_heads, head_dim, v_dim, q_weight, k_weight, w_is_f32, eps,
+                       positions, temp_coef, temp_every, slots, (elem_t*)k_cache, (elem_t*)v_cache, page_size);
     return nva_check_launch("qk_rownorm_store");
 }
 

@@ -394,7 +394,8 @@ class HipKernels:
         sum of the addends), then y = residual * rsqrt(mean(residual^2) + eps) * (offset + weight),
         all in float and rounded once.  addends: up to two tensors of the element type [rows, width].
         Returns (y, residual)."""
-        addends = [_t(a) for a in addends]
+        # a product left as partial sums is added up here, while it is read; anything else is a tensor
+        addends = [a if isinstance(a, SplitSum) and self.fuse_split_sums else _t(a) for a in addends]
         if len(addends) > 2 or (residual is None and not addends):
             raise KernelError("stream_rms_norm: one or two addends (none only with a stream that exists)")
         ref = addends[0] if addends else None
@@ -403,30 +404,33 @@ class HipKernels:
                 raise KernelError("stream_rms_norm: without addends the output tensor says the element type")
             rows, width = residual.shape
         else:
-            rows, width, _ = _rows2d(ref, "stream_rms_norm addend")
-        strides = []
+            rows, width = ref.shape
+        args = []
         for a in addends:
-            ar, aw, as_ = _rows2d(a, "stream_rms_norm addend")
-            if (ar, aw) != (rows, width) or a.dtype != ref.dtype:
+            if tuple(a.shape) != (rows, width) or a.dtype != ref.dtype:
                 raise KernelError("stream_rms_norm: the addends differ in shape or type")
-            strides.append(as_)
+            if isinstance(a, SplitSum):
+                args += [None, c_i64(0), _p(a.sums), c_i32(a.splits), c_i64(rows * width), _p(a.bias)]
+            else:
+                _, _, as_ = _rows2d(a, "stream_rms_norm addend")
+                args += [_p(a), c_i64(as_), None, c_i32(0), c_i64(0), None]
+        for _ in range(2 - len(addends)):
+            args += [None, c_i64(0), None, c_i32(0), c_i64(0), None]
         first = residual is None
+        device = ref.device if ref is not None else residual.device
         if first:
-            residual = torch.empty((rows, width), dtype=torch.float32, device=ref.device)
+            residual = torch.empty((rows, width), dtype=torch.float32, device=device)
         rrows, rw, rs = _rows2d(residual, "stream_rms_norm residual")
         if (rrows, rw) != (rows, width) or residual.dtype != torch.float32:
             raise KernelError("stream_rms_norm: the residual stream must be float32 of the addends' shape")
         dtype = ref.dtype if ref is not None else out.dtype
         if out is None:
-            out = torch.empty((rows, width), dtype=dtype, device=residual.device)
+            out = torch.empty((rows, width), dtype=dtype, device=device)
         orows, ow, os_ = _rows2d(out, "stream_rms_norm output")
         if (orows, ow) != (rows, width) or out.dtype != dtype:
             raise KernelError("stream_rms_norm: output does not match")
         wf = self._norm_weight(weight, width, out)
-        a = addends[0] if addends else None
-        b = addends[1] if len(addends) > 1 else None
-        library.call("norm", _suffix(out), "nva_stream_rms_norm", _p(a), c_i64(strides[0] if addends else 0), _p(b),
-                     c_i64(strides[1] if len(addends) > 1 else 0), _p(residual), c_i64(rs), c_i32(1 if first else 0),
+        library.call("norm", _suffix(out), "nva_stream_rms_norm", *args, _p(residual), c_i64(rs), c_i32(1 if first else 0),
                      _p(weight), c_i32(wf), c_f32(offset), _p(out), c_i64(os_), c_i64(rows), c_i32(width), c_f32(eps),
                      self._stream())
         return out, residual
@@ -914,8 +918,12 @@ class HipKernels:
         and [kv_heads * head_dim]), q scaled by the temperature 1 + temp_coef * ln(floor((p + 1) /
         temp_every) + 1) of its position p, both written back in place, k and v written into their page
         slots.  The row is [q | k | v] with values of v_head_dim.  Returns the q view."""
-        qkv = _t(qkv)
-        tokens, width, stride = _rows2d(qkv, "qkv")
+        partial = isinstance(qkv, SplitSum) and self.fuse_split_sums
+        if partial:
+            (tokens, width), stride = qkv.shape, 0
+        else:
+            qkv = _t(qkv)
+            tokens, width, stride = _rows2d(qkv, "qkv")
         want = (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_head_dim
         if width != want:
             raise KernelError(f"qkv width {width} is not heads * head_dim + kv_heads * (head_dim + v_head_dim) = {want}")
@@ -935,11 +943,19 @@ class HipKernels:
         if k_cache is not None:
             page_size = self._check_cache(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype, v_head_dim)
             _i32(slots, tokens, "slots")
-        library.call("qk_rownorm", _suffix(qkv), "nva_qk_rownorm_store", _p(qkv), c_i64(stride), c_i64(tokens),
+        if partial:
+            # the projection's partial sums (and bias) are added up by the kernel; q gets a tensor of its own
+            q = torch.empty((tokens, num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+            source = [None, c_i64(0), _p(qkv.sums), c_i32(qkv.splits), c_i64(tokens * width), _p(qkv.bias), _p(q),
+                      c_i64(num_heads * head_dim)]
+        else:
+            q = qkv[:, : num_heads * head_dim]
+            source = [_p(qkv), c_i64(stride), None, c_i32(0), c_i64(0), None, _p(qkv), c_i64(stride)]
+        library.call("qk_rownorm", "bf16" if partial else _suffix(qkv), "nva_qk_rownorm_store", *source, c_i64(tokens),
                      c_i32(num_heads), c_i32(num_kv_heads), c_i32(head_dim), c_i32(v_head_dim), _p(q_weight), _p(k_weight),
                      c_i32(wf), c_f32(eps), _p(positions), c_f32(float(temp_coef)), c_i32(int(temp_every) if temp_coef else 1),
                      _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size), self._stream())
-        return qkv[:, : num_heads * head_dim]
+        return q
 
     @staticmethod
     def _check_cache(k_cache, v_cache, num_kv_heads, head_dim, dtype, v_head_dim=None) -> int:

@@ -128,7 +128,7 @@ class Attention(Part):
         pe = self.position_encoding
         table = pe.rotary_table() if pe is not None else None
         qkv = k.linear(x, w["qkv_proj.weight"], w.get("qkv_proj.bias"),
-                       deferred=not self.row_prepare and (pe is None or table is not None))
+                       deferred=self.row_prepare or pe is None or table is not None)
         group = batch.groups[cache.group]
         slots = None if self.shared else group.slot_mapping
         kc, vc = (None, None) if self.shared else (cache.k, cache.v)
