@@ -132,6 +132,14 @@ __device__ __forceinline__ float nva_exp(float x) {
 #endif
 }
 
+// ---------------------------------------------------------------------------- gating
+// The activation of a gated feed-forward, by its code: 0 silu, 1 relu, 2 gelu (tanh form).
+__device__ __forceinline__ float nva_gate_act(int act, float g) {
+    if (act == 1) return fmaxf(g, 0.f);
+    if (act == 2) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return g / (1.f + __expf(-g));
+}
+
 // ---------------------------------------------------------------------------- split products
 // A product whose k range was split over workgroups leaves float partial sums
 // [splits][rows][width] (gemm_skinny.hip).  Kernels that consume such a product add the partials

@@ -69,7 +69,7 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
     const int k_end = min(K, k_begin + k_per_split);
     const int xs_stride = chunk + 8;
 
-    const bool gated = direct == 2;
+    const bool gated = direct >= 2;      // 2 + the activation's code (common.h: nva_gate_act)
     const int inner = N / 2;
     const int tile = blockIdx.x * (WAVES / KW) + wave / KW;
     const int ksub = wave % KW;
@@ -160,7 +160,7 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
                 const float gate = (float)(__bf16)acc[b][i];
                 const int j = n0 + 4 * g + i;
                 if (g < 2 && m < M && j < inner) {
-                    const float v = gate / (1.f + __expf(-gate)) * up;
+                    const float v = nva_gate_act(direct - 2, gate) * up;
                     if (y_is_f32) ((float*)y)[(int64_t)m * y_stride + j] = v;
                     else ((__bf16*)y)[(int64_t)m * y_stride + j] = (__bf16)v;
                 }
@@ -223,7 +223,7 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
     const int k_begin = split * k_per_split;
     const int k_end = min(K, k_begin + k_per_split);
     const int chunks = (k_end - k_begin + MD_KC - 1) / MD_KC;
-    const bool gated = direct == 2;
+    const bool gated = direct >= 2;      // 2 + the activation's code (common.h: nva_gate_act)
     const int inner = N / 2;
     const int per_tile = gated ? 8 : 16;
     const int tile0 = (blockIdx.x * WAVES + wave) * RT;
@@ -343,7 +343,7 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
                     const float gate = (float)(__bf16)acc[rt][b][i];
                     const int j = n0 + 4 * g + i;
                     if (g < 2 && m < M && j < inner) {
-                        const float v = gate / (1.f + __expf(-gate)) * up;
+                        const float v = nva_gate_act(direct - 2, gate) * up;
                         if (y_is_f32) ((float*)y)[(int64_t)m * y_stride + j] = v;
                         else ((__bf16*)y)[(int64_t)m * y_stride + j] = (__bf16)v;
                     }
@@ -403,7 +403,7 @@ linear_skinny_finish_kernel(const float* __restrict__ partial, int splits, const
         // the reference rounds the projection to bfloat16 before the gating (activation.py:8-11)
         v = (float)(__bf16)v;
         u = (float)(__bf16)u;
-        v = v / (1.f + __expf(-v)) * u;
+        v = nva_gate_act(swiglu - 1, v) * u;
     }
     if (y_is_f32) ((float*)y)[(int64_t)m * y_stride + j] = v;
     else ((__bf16*)y)[(int64_t)m * y_stride + j] = (__bf16)v;
@@ -427,12 +427,12 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
     if (waves_per_tile != 1 && waves_per_tile != 2 && waves_per_tile != 4)
         return nva_fail("linear_skinny: 1, 2 or 4 waves share rows of W, not %d", waves_per_tile);
     if (swiglu && (N % 2)) return nva_fail("linear_skinny: the gated form needs an even number of weight rows");
-    const int direct = splits == 1 && !bias && !defer_finish ? (swiglu ? 2 : 1) : 0;
+    const int direct = splits == 1 && !bias && !defer_finish ? (swiglu ? 1 + swiglu : 1) : 0;
     if (!direct && !scratch) return nva_fail("linear_skinny: this call needs scratch memory");
     int kps = (int)((K + splits - 1) / splits);
     kps = (kps + SK_KSTEP * SK_UNROLL - 1) / (SK_KSTEP * SK_UNROLL) * (SK_KSTEP * SK_UNROLL);
     const int real_splits = (int)((K + kps - 1) / kps);
-    const int64_t tiles = direct == 2 ? (N / 2 + 7) / 8 : (N + 15) / 16;
+    const int64_t tiles = direct >= 2 ? (N / 2 + 7) / 8 : (N + 15) / 16;
     // columns of x staged at a time: about 36 KB of LDS for the M + 1 rows, so that several workgroups fit a CU
     int chunk = (36864 / (2 * ((int)M + 1)) - 8) / 256 * 256;
     chunk = chunk < 256 ? 256 : chunk > 2048 ? 2048 : chunk;
@@ -487,12 +487,12 @@ NVA_EXPORT int nva_linear_medium_bf16(const void* x, int64_t x_stride, const voi
     if (row_tiles < 1 || row_tiles > 3 || (row_tiles == 3 && mb > 6) || (row_tiles == 2 && mb > 14) || (waves == 3 && mb > 6))
         return nva_fail("linear_medium: %d row tiles per wave and %d waves are not built for %lld rows", row_tiles, waves, (long long)M);
     if (swiglu && (N % 2)) return nva_fail("linear_medium: the gated form needs an even number of weight rows");
-    const int direct = splits == 1 && !bias && !defer_finish ? (swiglu ? 2 : 1) : 0;
+    const int direct = splits == 1 && !bias && !defer_finish ? (swiglu ? 1 + swiglu : 1) : 0;
     if (!direct && !scratch) return nva_fail("linear_medium: this call needs scratch memory");
     int kps = (int)((K + splits - 1) / splits);
     kps = (kps + MD_KC - 1) / MD_KC * MD_KC;
     const int real_splits = (int)((K + kps - 1) / kps);
-    const int64_t tiles = direct == 2 ? (N / 2 + 7) / 8 : (N + 15) / 16;
+    const int64_t tiles = direct >= 2 ? (N / 2 + 7) / 8 : (N + 15) / 16;
     const size_t lds = (size_t)2 * (16 * mb + 1) * MD_XS * sizeof(__bf16);
 #define LAUNCH(MB, RT, WV)                                                                                             \
     do {                                                                                                               \

@@ -27,7 +27,7 @@ enum { TM_PLAIN = 0, TM_PLAIN_F32 = 1, TM_GATED = 2 };
 struct TeamArgs {
     const __bf16* x; int64_t x_stride;
     const __bf16* w; int64_t w_stride; const __bf16* bias;
-    void* y; int64_t y_stride; int mode;
+    void* y; int64_t y_stride; int mode; int act;
     int M, N, K, blocks, blocks_per_team, frags_per_wave;
 };
 
@@ -147,7 +147,7 @@ linear_team_kernel(const TeamArgs a) {
                     const float gate = round_through<__bf16>(v[i]);
                     const int j = blk * 8 + 4 * g + i;
                     if (g < 2 && m < a.M && j < inner)
-                        ((__bf16*)a.y)[(int64_t)m * a.y_stride + j] = (__bf16)(gate / (1.f + __expf(-gate)) * up);
+                        ((__bf16*)a.y)[(int64_t)m * a.y_stride + j] = (__bf16)(nva_gate_act(a.act, gate) * up);
                 }
                 continue;
             }
@@ -179,12 +179,15 @@ NVA_EXPORT int nva_linear_team_bf16(const void* x, int64_t x_stride, const void*
     }
     if (teams <= 0 || !x || !w || !y || x_stride % 8 || w_stride % 8 || !nva_aligned(x, 16) || !nva_aligned(w, 16))
         return nva_fail("linear_team: x and W need 16-byte aligned rows, and an output");
-    if (mode < 0 || mode > 2) return nva_fail("linear_team: unknown mode %d", mode);
+    // modes 2, 3, 4: the gated form with silu, relu, gelu (tanh)
+    if (mode < 0 || mode > 4) return nva_fail("linear_team: unknown mode %d", mode);
+    const int act = mode > TM_GATED ? mode - TM_GATED : 0;
+    if (mode > TM_GATED) mode = TM_GATED;
     if (mode == TM_GATED && (N % 2 || bias)) return nva_fail("linear_team: the gated form needs an even number of weight rows and no bias");
     TeamArgs a;
     a.x = (const __bf16*)x; a.x_stride = x_stride;
     a.w = (const __bf16*)w; a.w_stride = w_stride; a.bias = (const __bf16*)bias;
-    a.y = y; a.y_stride = y_stride; a.mode = mode;
+    a.y = y; a.y_stride = y_stride; a.mode = mode; a.act = act;
     a.M = (int)M; a.N = (int)N; a.K = (int)K;
     a.blocks = mode == TM_GATED ? (int)((N / 2 + 7) / 8) : (int)((N + 15) / 16);
     a.blocks_per_team = (a.blocks + teams - 1) / teams;

@@ -35,7 +35,7 @@ enum { TL_PLAIN = 0, TL_PLAIN_F32 = 1, TL_GATED = 2, TL_PARTIAL = 3 };
 struct TileArgs {
     const __bf16* x; int64_t x_stride;
     const __bf16* w; int64_t w_stride; const __bf16* bias;
-    void* y; int64_t y_stride; float* partial; int mode;
+    void* y; int64_t y_stride; float* partial; int mode; int act;
     int M, N, K, chunks_per_range;
     int cols_per_wg;        // columns of y a workgroup takes: those of its tile, or fewer (the tile's other rows of W are not fetched)
 };
@@ -112,7 +112,7 @@ __device__ __forceinline__ void tile_store(const TileArgs& a, const f32x16 (&acc
                         const float gate = round_through<__bf16>(acc[tm][tn][v]);
                         const float up = round_through<__bf16>(acc[tm][tn + TN / 2][v]);
                         if (m < a.M && j < min(inner, n0 + a.cols_per_wg))
-                            ((__bf16*)a.y)[(int64_t)m * a.y_stride + j] = (__bf16)(gate / (1.f + __expf(-gate)) * up);
+                            ((__bf16*)a.y)[(int64_t)m * a.y_stride + j] = (__bf16)(nva_gate_act(a.act, gate) * up);
                     }
         }
         return;
@@ -344,7 +344,10 @@ NVA_EXPORT int nva_linear_tile_bf16(const void* x, int64_t x_stride, const void*
     }
     if (!x || !w || x_stride % 8 || w_stride % 8 || !nva_aligned(x, 16) || !nva_aligned(w, 16))
         return nva_fail("linear_tile: x and W need 16-byte aligned rows");
-    if (mode < 0 || mode > 3) return nva_fail("linear_tile: unknown mode %d", mode);
+    // modes 4, 5: the gated form with relu, gelu (tanh); 2 is silu
+    if (mode < 0 || mode > 5) return nva_fail("linear_tile: unknown mode %d", mode);
+    const int act = mode > TL_PARTIAL ? mode - TL_PARTIAL : 0;
+    if (mode > TL_PARTIAL) mode = TL_GATED;
     if (shape < 0 || shape >= nva_linear_tile_shapes()) return nva_fail("linear_tile: unknown tile shape %d", shape);
     const TileShapeInfo sh = tile_shapes[shape];
     if (mode == TL_GATED && (N % 2 || bias)) return nva_fail("linear_tile: the gated form needs an even number of weight rows and no bias");
@@ -362,7 +365,7 @@ NVA_EXPORT int nva_linear_tile_bf16(const void* x, int64_t x_stride, const void*
     TileArgs a;
     a.x = (const __bf16*)x; a.x_stride = x_stride;
     a.w = (const __bf16*)w; a.w_stride = w_stride; a.bias = (const __bf16*)bias;
-    a.y = y; a.y_stride = y_stride; a.partial = partial; a.mode = mode;
+    a.y = y; a.y_stride = y_stride; a.partial = partial; a.mode = mode; a.act = act;
     a.M = (int)M; a.N = (int)N; a.K = (int)K;
     const int chunks = (int)(K / TL_BK);
     a.chunks_per_range = (chunks + ranges - 1) / ranges;

@@ -459,13 +459,6 @@ class HipKernels:
     def silu_mul(self, gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         return self.act_mul(gate_up, "silu", out=out)
 
-    def linear_act_mul(self, x: torch.Tensor, weight: torch.Tensor, act: str = "silu") -> torch.Tensor:
-        """act(x @ Wg.T) * (x @ Wu.T) with weight = [Wg; Wu].  silu has the gating in the products'
-        epilogues (linear_silu_mul); the other activations run the product and the gating kernel."""
-        if act == "silu":
-            return self.linear_silu_mul(x, weight)
-        return self.act_mul(self.linear(x, weight), act)
-
     # ------------------------------------------------------------------ matrix products
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                out_float32: bool = False, out: Optional[torch.Tensor] = None, deferred: bool = False):
@@ -677,7 +670,7 @@ class HipKernels:
         used = ctypes.c_int(0)
         library.call("gemm_skinny", "bf16", "nva_linear_skinny", _p(x), c_i64(xs), _p(weight), c_i64(ws),
                      None if defer else _p(bias), _p(out), c_i64(os_), c_i32(1 if out_float32 else 0),
-                     c_i32(1 if swiglu else 0), _p(scratch), c_i32(splits), c_i32(kw), c_i32(1 if defer else 0), c_i64(m), c_i64(n),
+                     c_i32(int(swiglu)), _p(scratch), c_i32(splits), c_i32(kw), c_i32(1 if defer else 0), c_i64(m), c_i64(n),
                      c_i64(k), ctypes.byref(used), self._stream())
         if defer:
             return SplitSum(self, scratch, used.value, m, n, bias)
@@ -729,7 +722,7 @@ class HipKernels:
         used = ctypes.c_int(0)
         library.call("gemm_skinny", "bf16", "nva_linear_medium", _p(x), c_i64(xs), _p(weight), c_i64(ws),
                      None if defer else _p(bias), _p(out), c_i64(os_), c_i32(1 if out_float32 else 0),
-                     c_i32(1 if swiglu else 0), _p(scratch), c_i32(splits), c_i32(rt), c_i32(waves), c_i32(1 if defer else 0),
+                     c_i32(int(swiglu)), _p(scratch), c_i32(splits), c_i32(rt), c_i32(waves), c_i32(1 if defer else 0),
                      c_i64(m), c_i64(n), c_i64(k), ctypes.byref(used), self._stream())
         if defer:
             return SplitSum(self, scratch, used.value, m, n, bias)
@@ -786,7 +779,8 @@ class HipKernels:
                 defer = False
                 out = torch.empty((m, n), dtype=x.dtype, device=x.device)
                 os_ = n
-            mode = 2 if gated else 1 if out_float32 else 0
+            # (the gated form by its activation: swiglu is True or 1 for silu, 2 relu, 3 gelu)
+            mode = (2 if int(swiglu) == 1 else 2 + int(swiglu)) if gated else 1 if out_float32 else 0
             library.call("gemm_tile", "bf16", "nva_linear_tile", _p(x), c_i64(xs), _p(weight), c_i64(ws), _p(bias), _p(out),
                          c_i64(os_), None, c_i32(mode), c_i64(m), c_i64(n), c_i64(k), c_i32(shape), c_i32(stages), c_i32(1),
                          c_i32(cols), None, self._stream())
@@ -811,13 +805,21 @@ class HipKernels:
 
     def linear_silu_mul(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         """silu(x @ Wg.T) * (x @ Wu.T) with weight = [Wg; Wu]."""
+        return self.linear_act_mul(x, weight, "silu")
+
+    def linear_act_mul(self, x: torch.Tensor, weight: torch.Tensor, act: str = "silu") -> torch.Tensor:
+        """act(x @ Wg.T) * (x @ Wu.T) with weight = [Wg; Wu]; act: silu, relu or gelu_tanh.  The product
+        kernels do the gating in their epilogues, whatever the activation."""
+        if act not in self.ACTIVATIONS:
+            raise KernelError(f"linear_act_mul: unknown activation {act!r}; known: {sorted(self.ACTIVATIONS)}")
+        code = self.ACTIVATIONS[act]            # the kernels' gating flag is 1 + code, the team kernel's mode 2 + code
         x = _t(x)
         m, k, xs = _rows2d(x, "linear input")
         n, wk, ws = _rows2d(weight, "linear weight")
         if x.dtype == torch.bfloat16 and weight.dtype == x.dtype and wk == k and n % 2 == 0 and \
                 self._own_kernel(m, n, k) == "team" and self._skinny_takes(x, xs, weight, ws, k):
             out = torch.empty((m, n // 2), dtype=x.dtype, device=x.device)
-            return self._linear_team(x, xs, weight, ws, None, out, n // 2, 2, m, n, k)
+            return self._linear_team(x, xs, weight, ws, None, out, n // 2, 2 + code, m, n, k)
         if x.dtype == torch.bfloat16 and weight.dtype == x.dtype and wk == k and n % 2 == 0 and \
                 self._skinny_takes(x, xs, weight, ws, k):
             own = self._own_kernel(m, n, k, gated=True)
@@ -826,11 +828,11 @@ class HipKernels:
             if own in ("skinny", "medium", "tile"):
                 out = torch.empty((m, n // 2), dtype=x.dtype, device=x.device)
                 run = self._linear_skinny if own == "skinny" else self._linear_medium if own == "medium" else self._linear_tile
-                run(x, xs, weight, ws, None, out, n // 2, False, True, m, n, k)
+                run(x, xs, weight, ws, None, out, n // 2, False, 1 + code, m, n, k)
                 return out
             if m > self.own_matmul_rows and (n, k, True) in self.product_choice:
-                return self.silu_mul(torch.nn.functional.linear(x, weight))      # measured: the library here
-        return self.silu_mul(self.linear(x, weight))
+                return self.act_mul(torch.nn.functional.linear(x, weight), act)      # measured: the library here
+        return self.act_mul(self.linear(x, weight), act)
 
     # ------------------------------------------------------------------ position encoding
     def rotary_table(self, inv_freq: torch.Tensor, num_positions: int) -> torch.Tensor:

@@ -132,6 +132,22 @@ def test_gating_with_each_activation(backend, dtype):
             _close(k.act_mul(x.to(dev), act), w, dtype, act)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("act", ["relu", "gelu_tanh", "silu"])
+def test_gated_products_with_each_activation_at_every_row_count(act):
+    # the product kernels gate in their epilogues: every kernel that a row count and a weight's shape
+    # select, against the product and the gating done apart in float
+    k, dev = _kernels("hip", torch.bfloat16)
+    g = torch.Generator().manual_seed(11)
+    for inner, width in ((96, 64), (1536, 512), (5120, 256)):
+        w = (torch.randn((2 * inner, width), generator=g) / math.sqrt(width)).to(torch.bfloat16).to(dev)
+        for rows in (1, 3, 8, 16, 40, 130, 256, 300):
+            x = torch.randn((rows, width), generator=g).to(torch.bfloat16).to(dev)
+            got = k.linear_act_mul(x, w, act)
+            want = TorchKernels(dev, torch.bfloat16).linear_act_mul(x, w, act)
+            _close(got, want.cpu(), torch.bfloat16, f"{act} inner {inner} rows {rows}")
+
+
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("hq,hkv,D,DV,page,every", [(6, 2, 16, 24, 8, 5), (4, 4, 24, 24, 16, 1), (3, 1, 40, 16, 4, 7)])
