@@ -183,7 +183,7 @@ NVA_EXPORT int NVA_NAME(nva_rms_norm_of_partials)(const float* sums, int splits,
 // An addend may be given as the float partial sums of a product whose k range was split (pa, pb): they
 // are added, with the bias, and rounded to the element type as the product's own finishing pass would.
 template <typename T>
-__global__ void __launch_bounds__(512)
+__global__ void __launch_bounds__(1024)
 stream_rms_norm_kernel(const T* __restrict__ a, int64_t a_stride, PartialInput pa, const T* __restrict__ b,
                        int64_t b_stride, PartialInput pb, float* residual, int64_t r_stride, int first,
                        const void* __restrict__ weight, int w_is_f32, float offset, T* __restrict__ y,
@@ -239,7 +239,9 @@ NVA_EXPORT int NVA_NAME(nva_stream_rms_norm)(const void* a, int64_t a_stride, co
     if ((a_sums && (a_splits <= 0 || a_split_stride < rows * (int64_t)width)) ||
         (b_sums && (b_splits <= 0 || b_split_stride < rows * (int64_t)width)))
         return nva_fail("stream_rms_norm: bad partial sums");
-    const int threads = width >= 2048 ? 512 : width >= 1024 ? 256 : width >= 256 ? 128 : 64;
+    // (partial sums of few rows: an element a thread, so that a row's sums are asked for at once)
+    const int threads = (a_sums || b_sums) && rows <= 64 && width >= 1024 ? 1024
+                        : width >= 2048 ? 512 : width >= 1024 ? 256 : width >= 256 ? 128 : 64;
     hipLaunchKernelGGL((stream_rms_norm_kernel<elem_t>), dim3((unsigned)rows), dim3(threads), 0, stream,
                        (const elem_t*)a, a_stride, pa, (const elem_t*)b, b_stride, pb, residual, r_stride, first, weight,
                        w_is_f32, offset, (elem_t*)y, y_stride, width, eps);

@@ -17,7 +17,7 @@
 #include "common.h"
 
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput part, T* __restrict__ q_out,
                         int64_t q_stride, int num_heads, int num_kv_heads, int head_dim, int v_dim,
                         const void* __restrict__ q_weight, const void* __restrict__ k_weight, int w_is_f32, float eps,
@@ -107,7 +107,9 @@ NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(const void* qkv, int64_t stride, c
         raised = true;
     }
     const PartialInput part{sums, splits, split_stride, bias};
-    hipLaunchKernelGGL(kernel, dim3((unsigned)tokens), dim3(256), lds, stream, (const elem_t*)qkv, stride, part,
+    // few tokens (a decode step): more threads a token, so that a row of partial sums is asked for at once
+    const int threads = tokens <= 64 && width >= 2048 ? 1024 : 256;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)tokens), dim3(threads), lds, stream, (const elem_t*)qkv, stride, part,
                        (elem_t*)q_out, q_stride, num_heads, num_kv_heads, head_dim, v_dim, q_weight, k_weight, w_is_f32, eps,
                        positions, temp_coef, temp_every, slots, (elem_t*)k_cache, (elem_t*)v_cache, page_size);
     return nva_check_launch("qk_rownorm_store");
