@@ -1,5 +1,6 @@
 """Named config.json contents for runs with random weights (there is no checkpoint to read
-them from): two tiny test shapes and the Qwen3 dense sizes that the benchmarks use.  These are
+them from): two tiny test shapes and the Qwen3 dense sizes that the benchmarks use, and three
+Nozurax shapes (a tiny one, and layers of the Qwen3 1.7B and 8B sizes).  These are
 inputs, as a model folder's config.json is; nothing in the model code reads them.
 
     python -m nano_vllm_amd.cli random-model --shape qwen3-8b --config-only --out DIR
@@ -19,7 +20,28 @@ def _qwen3(layers, hidden, heads, kv_heads, head_dim, inner, vocab, theta=1e6, e
             "hidden_act": "silu", "torch_dtype": dtype}
 
 
+def _nozurax(layers, width, heads, kv_heads, dim, vdim, inner, vocab, eps=1e-6, every=256, dtype="bfloat16",
+             ret_heads=None, rot=None, pattern=("attention", "retention")) -> dict:
+    """Layers that follow `pattern` in turn, each with tensors of its own: attention (sinks, whole-projection
+    norms, a query temperature) and retention (decays 1 - 2^-5 ... 1 - 2^-8 over the heads, rotation of `rot`
+    channels, default the whole head)."""
+    rh = ret_heads or heads
+    kinds = {
+        "attention": {"type": "attention", "mlp": {"kind": "dense", "ff": inner},
+                      "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
+                                "q_temp": {"coef": 0.1, "every": every}}},
+        "retention": {"type": "retention", "mlp": {"kind": "dense", "ff": inner},
+                      "mixer": {"heads": rh, "dim": dim, "vdim": vdim, "rot": {"dims": rot or dim, "base": 1e6},
+                                "decay": [1.0 - 2.0 ** (-5 - 3.0 * h / rh) for h in range(rh)]}},
+    }
+    return {"architecture": "Nozurax", "vocab": vocab, "width": width, "norm": {"eps": eps},
+            "layers": [kinds[pattern[i % len(pattern)]] for i in range(layers)], "torch_dtype": dtype}
+
+
 SHAPES: Dict[str, dict] = {
+    "nozurax-tiny": _nozurax(4, 64, 4, 2, 16, 24, 96, 256, eps=1e-5, every=8, dtype="float32", ret_heads=2, rot=8),
+    "nozurax-1b": _nozurax(16, 2048, 16, 8, 128, 128, 6144, 32768),
+    "nozurax-8b": _nozurax(32, 4096, 32, 8, 128, 128, 12288, 32768),
     "tiny-a": _qwen3(2, 64, 4, 2, 16, 128, 256, theta=1e4, tied=True, max_position=128, dtype="float32"),
     "tiny-b": _qwen3(3, 96, 8, 2, 32, 160, 384, eps=1e-5, max_position=256, dtype="float32"),
     "qwen3-0.6b": _qwen3(28, 1024, 16, 8, 128, 3072, 151936, tied=True),     # the model of the reference's README benchmark

@@ -10,6 +10,10 @@ def test_named_shapes_are_valid_configurations():
     for name in SHAPES:
         cj = shape(name)
         cfg = architecture_of(cj).parse_config(cj)
+        if name.startswith("nozurax"):
+            assert cfg.to_dict()["width"] == cj["width"] and len(cfg.layers) == len(cj["layers"])
+            assert architecture_of(cfg.to_dict()).parse_config(cfg.to_dict()) == cfg
+            continue
         assert cfg.num_attention_heads % cfg.num_key_value_heads == 0
         assert cfg.to_dict()["hidden_size"] == cj["hidden_size"]
     big = architecture_of(shape("qwen3-8b")).parse_config(shape("qwen3-8b"))
@@ -23,6 +27,10 @@ def test_random_model_command_writes_a_shape(tmp_path, capsys):
     assert main(["random-model", "--shape", "tiny-b", "--seed", "2", "--out", str(tmp_path / "m")]) == 0
     assert (tmp_path / "m" / "model.safetensors").exists()
     assert main(["random-model", "--out", str(tmp_path / "x")]) == 2
+    assert main(["random-model", "--shape", "nozurax-tiny", "--seed", "3", "--out", str(tmp_path / "n")]) == 0
+    from safetensors.torch import load_file
+    names = set(load_file(str(tmp_path / "n" / "model.safetensors")))
+    assert {"embed", "head", "final.norm", "l0.mix.sink", "l1.mix.g", "l3.mlp.down"} <= names
 
 
 def test_throughput_command_refuses_an_empty_range_of_lengths(capsys):
