@@ -290,6 +290,30 @@ def test_attention_with_a_sink_reads_a_far_key_among_hundreds(backend, dtype):
         assert float((got - want).abs().max()) < 0.05
 
 
+@pytest.mark.gpu
+def test_sinks_in_the_matrix_core_kernels_over_long_contexts():
+    # single tokens whose keys are shared out over many waves and merged, and a long portion: the
+    # matrix-core kernels against the general ones, and both against the dense softmax
+    k, dev = _kernels("hip", torch.bfloat16)
+    hq, hkv, D, page = 8, 2, 128, 64
+    lens, q_lens = [3000, 5000, 700], [1, 1, 260]
+    q, kc, vc, batch, (qs, ks, vs) = _sink_case(torch.bfloat16, dev, hq, hkv, D, D, page, lens, q_lens, seed=9)
+    sinks = torch.linspace(-2.0, 6.0, hq)
+    fast = k.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, D ** -0.5, None, v_head_dim=D, sinks=sinks.to(dev)).float().cpu()
+    k.mfma_attention = False
+    try:
+        general = k.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, D ** -0.5, None, v_head_dim=D, sinks=sinks.to(dev)).float().cpu()
+    finally:
+        k.mfma_attention = True
+    want = _sink_softmax(qs, ks, vs, lens, q_lens, D ** -0.5, sinks)
+    assert float((general.double() - want).abs().max()) < 1e-2
+    assert float((fast.double() - want).abs().max()) < 2e-2
+    # the sink's share is visible: without it the outputs are larger
+    none = k.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, D ** -0.5, None).float().cpu()
+    assert float((none - fast).abs().max()) > 5e-3
+    k.check_faults()
+
+
 def _retention_inputs(heads, dim, vdim, T, seed, dtype):
     g = torch.Generator().manual_seed(seed)
     hidden = heads * vdim
@@ -345,6 +369,7 @@ def _retention_constants(k, dev, decay, dim, rot, base):
     (2, 128, 160, (0.9, 0.999), 64, 1e6),
     (1, 256, 32, (0.99,), 0, 0.0),
     (3, 96, 96, (0.5, 1.0, 0.75), 96, 100.0),
+    (2, 32, 64, (0.9, 0.99), 8, 100.0),         # a rotation too narrow for the loads of eight elements
 ])
 def test_retention_in_portions_of_every_size_and_token_by_token(backend, dtype, heads, dim, vdim, decay, rot, base):
     k, dev = _kernels(backend, dtype)
@@ -587,6 +612,32 @@ def test_greedy_generation_through_the_engine(backend, schedule):
     for p, o in zip(prompts, outs):
         assert o["token_ids"] == plain.greedy_generate(cfg, w, p, 12), len(p)
     assert llm.runner.cache.slots.num_free == 3 and llm.runner.cache.pools[0].num_free == 10
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_models_of_one_kind_of_layer_and_tensors_owned_by_a_later_layer(backend, tmp_path):
+    # retention only (no pages at all), attention only (no state slots), and an entry that runs the
+    # tensors of a layer further down the list; layers without a feed-forward among them
+    from nano_vllm_amd.weights import write_random_model
+    cases = {
+        "retention": NozuraxConfig(vocab=120, width=40, eps=1e-6, layers=(
+            N._ret(0, 2, 8, 12, (0.9, 0.99), rot=8, base=1e4, ff=None), N._ret(1, 1, 16, 8, (0.95,), ff=56))),
+        "attention": NozuraxConfig(vocab=120, width=40, eps=1e-6, layers=(
+            N._att(0, 4, 1, 8, 12, 0.3, ff=None), N._att(1, 2, 2, 16, 8, 0.2, coef=0.4, every=2, ff=48))),
+        "later": NozuraxConfig(vocab=90, width=24, eps=1e-5, layers=(
+            N._ret(0, 2, 8, 4, (0.9, 0.99), rot=4, base=10.0, ff=32, of=2), N._att(1, 2, 1, 8, 4, 0.3, coef=0.4, every=2, ff=None),
+            N._ret(2, 2, 8, 4, (0.9, 0.99), rot=4, base=10.0, ff=32))),
+    }
+    kernels, dev = _kernels(backend)
+    for name, cfg in cases.items():
+        folder = write_random_model(str(tmp_path / name), cfg, seed=3, std=0.2, dtype="float32")
+        c, w = plain.read_folder(folder)
+        prompts = [H.random_tokens(cfg.vocab, n, 5 + n) for n in (1, 19, 40)]
+        llm = LLM(folder, kernels=kernels, device=dev, dtype="float32", kvcache_block_size=8, num_kvcache_blocks=12,
+                  max_num_batched_tokens=16, max_num_seqs=2, schedule="mixed", max_model_len=96)
+        outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True), use_tqdm=False)
+        for p, o in zip(prompts, outs):
+            assert o["token_ids"] == plain.greedy_generate(c, w, p, 8), (name, len(p))
 
 
 @pytest.mark.gpu
