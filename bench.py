@@ -75,7 +75,7 @@ def design_configs(width: int, layers: int, dtype: str):
                      "q_temp": {"coef": 0.1, "every": 256}}}
     ret = {"type": "retention", "mlp": {"kind": "dense", "ff": inner},
            "mixer": {"heads": heads, "dim": dim, "vdim": dim, "rot": {"dims": dim, "base": 1e6},
-                     "decay": [1.0 - 2.0 ** (-5 - 3.0 * h / heads) for h in range(heads)]}}
+                     "decay": [1.0 - 2.0 ** (-6 - 4.0 * h / heads) for h in range(heads)]}}
     nozurax = {"architecture": "Nozurax", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6},
                "layers": [att if i % 2 == 0 else ret for i in range(layers)], "torch_dtype": dtype}
     qwen3 = {"architectures": ["Qwen3ForCausalLM"], "hidden_size": width, "num_hidden_layers": layers,

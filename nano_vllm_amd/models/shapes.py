@@ -23,7 +23,7 @@ def _qwen3(layers, hidden, heads, kv_heads, head_dim, inner, vocab, theta=1e6, e
 def _nozurax(layers, width, heads, kv_heads, dim, vdim, inner, vocab, eps=1e-6, every=256, dtype="bfloat16",
              ret_heads=None, rot=None, pattern=("attention", "retention")) -> dict:
     """Layers that follow `pattern` in turn, each with tensors of its own: attention (sinks, whole-projection
-    norms, a query temperature) and retention (decays 1 - 2^-5 ... 1 - 2^-8 over the heads, rotation of `rot`
+    norms, a query temperature) and retention (decays 1 - 2^-6 ... 1 - 2^-10 over the heads, rotation of `rot`
     channels, default the whole head)."""
     rh = ret_heads or heads
     kinds = {
@@ -32,7 +32,7 @@ def _nozurax(layers, width, heads, kv_heads, dim, vdim, inner, vocab, eps=1e-6, 
                                 "q_temp": {"coef": 0.1, "every": every}}},
         "retention": {"type": "retention", "mlp": {"kind": "dense", "ff": inner},
                       "mixer": {"heads": rh, "dim": dim, "vdim": vdim, "rot": {"dims": rot or dim, "base": 1e6},
-                                "decay": [1.0 - 2.0 ** (-5 - 3.0 * h / rh) for h in range(rh)]}},
+                                "decay": [1.0 - 2.0 ** (-6 - 4.0 * h / rh) for h in range(rh)]}},
     }
     return {"architecture": "Nozurax", "vocab": vocab, "width": width, "norm": {"eps": eps},
             "layers": [kinds[pattern[i % len(pattern)]] for i in range(layers)], "torch_dtype": dtype}

@@ -46,9 +46,9 @@ CONFIGS: Dict[str, dict] = {
     # sizes of the matrix-core attention's kind (equal head sizes of 64), so that whatever serves
     # them is compared with the general kernels
     "r": dict(cfg=NozuraxConfig(vocab=512, width=128, eps=1e-6, layers=(
-        _att(0, 8, 2, 64, 64, 0.125, coef=0.5, every=16, ff=192),
-        _ret(1, 2, 64, 64, (0.96875, 0.998), rot=64, base=1e4, ff=192),
-        _att(2, 8, 2, 64, 64, 0.125, coef=0.5, every=16, ff=192, of=0))), page=32, seed=23),
+        _att(0, 8, 2, 64, 64, 0.11, coef=0.4, every=16, ff=192),
+        _ret(1, 2, 64, 64, (0.95, 0.998), rot=64, base=1e4, ff=192),
+        _att(2, 8, 2, 64, 64, 0.11, coef=0.4, every=16, ff=192, of=0))), page=32, seed=23),
     "s": dict(cfg=NozuraxConfig(vocab=97, width=20, eps=1e-6, layers=(
         _ret(0, 2, 6, 10, (0.8, 0.99), rot=4, base=50.0, ff=28),
         _att(1, 2, 1, 6, 10, 0.4, coef=0.2, every=3, ff=28))), page=4, seed=24),

@@ -362,10 +362,10 @@ def _retention_constants(k, dev, decay, dim, rot, base):
     (3, 16, 8, (0.5, 0.9, 0.999), 8, 100.0),
     (1, 32, 32, (0.9375,), 32, 1e6),
     (2, 24, 40, (0.97, 1.0), 0, 0.0),
-    (2, 64, 72, (0.96875, 0.998), 64, 1e4),
+    (2, 64, 72, (0.95, 0.998), 64, 1e4),
     (2, 6, 10, (0.0, 0.99), 4, 50.0),
     # heads and values of multiples of 32 channels: the kernel on the matrix cores
-    (2, 64, 64, (0.96875, 0.998), 64, 1e4),
+    (2, 64, 64, (0.93, 0.9975), 64, 1e4),
     (2, 128, 160, (0.9, 0.999), 64, 1e6),
     (1, 256, 32, (0.99,), 0, 0.0),
     (3, 96, 96, (0.5, 1.0, 0.75), 96, 100.0),
