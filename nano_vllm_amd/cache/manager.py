@@ -28,8 +28,24 @@ from .pages import OutOfPages, PageError, PagePool, SlotPool
 
 @dataclass(frozen=True)
 class CacheGroup:
-    window: Optional[int]          # None: all keys
+    window: Optional[int]          # None: no window
     runs: Tuple[int, ...]          # entries of the model's order that keep their cache here
+    chunk: Optional[int] = None    # None: no chunks; else a query reads keys of its own chunk of positions only
+
+    @property
+    def reach(self) -> Optional[int]:
+        """How many positions back a query can read at most (itself included); None: all of them."""
+        bounds = [b for b in (self.window, self.chunk) if b is not None]
+        return min(bounds) if bounds else None
+
+    def first_key(self, query: int) -> int:
+        """The first position that a query at position `query` reads."""
+        lo = 0
+        if self.window is not None:
+            lo = max(lo, query - self.window + 1)
+        if self.chunk is not None:
+            lo = max(lo, query // self.chunk * self.chunk)
+        return lo
 
 
 @dataclass
@@ -45,19 +61,21 @@ def plan_groups(needs) -> Tuple[List[CacheGroup], List[int]]:
     """From the per-run needs (PagedKV / FixedState / None) the page groups, and the runs
     that keep fixed state.  A need is recognised by its attributes, so that this module
     imports nothing from the parts."""
-    by_window: Dict[Optional[int], List[int]] = {}
+    by_reach: Dict[Tuple[Optional[int], Optional[int]], List[int]] = {}
     state_runs: List[int] = []
     for i, need in enumerate(needs):
         if need is None:
             continue
-        if hasattr(need, "tensors"):
-            state_runs.append(i)
-        elif hasattr(need, "num_kv_heads"):
-            by_window.setdefault(need.window, []).append(i)
-        else:
-            raise ValueError(f"run {i}: unknown cache need {need!r}")
-    keys = sorted(by_window, key=lambda w: (w is not None, w or 0))       # the all-keys group first
-    return [CacheGroup(w, tuple(by_window[w])) for w in keys], state_runs
+        for part in getattr(need, "parts", (need,)):          # a combined need: pages and state for one run
+            if hasattr(part, "tensors"):
+                state_runs.append(i)
+            elif hasattr(part, "num_kv_heads"):
+                by_reach.setdefault((part.window, getattr(part, "chunk", None)), []).append(i)
+            else:
+                raise ValueError(f"run {i}: unknown cache need {part!r}")
+    # the all-keys group first, then by window and chunk
+    keys = sorted(by_reach, key=lambda wc: (wc != (None, None), wc[0] or 0, wc[1] or 0))
+    return [CacheGroup(w, tuple(by_reach[(w, c)]), c) for w, c in keys], state_runs
 
 
 def chain_hash(tokens: Sequence[int], prefix: int = -1) -> int:
@@ -111,15 +129,12 @@ class CacheManager:
 
     # ------------------------------------------------------------------ pages for new tokens
     def _first_needed_page(self, group: int, first_query: int) -> int:
-        w = self.groups[group].window
-        if w is None:
-            return 0
-        return max(0, first_query - w + 1) // self.page_size
+        return self.groups[group].first_key(first_query) // self.page_size
 
     def _wanted_pages(self, group: int, new_len: int, step_end: Optional[int]) -> int:
         """The length of the group's block table that covers positions < new_len; a window group
         covers only positions < step_end, the end of the step at hand, when that is given."""
-        if step_end is not None and self.groups[group].window is not None:
+        if step_end is not None and self.groups[group].reach is not None:
             new_len = min(new_len, step_end)
         return (new_len + self.page_size - 1) // self.page_size
 
@@ -145,10 +160,10 @@ class CacheManager:
         total = (num_tokens + self.page_size - 1) // self.page_size
         out = []
         for group in self.groups:
-            if group.window is None:
+            if group.reach is None:
                 out.append(total)
             else:
-                span = group.window - 1 + max(1, min(portion, num_tokens))       # positions a step touches, at any offset
+                span = group.reach - 1 + max(1, min(portion, num_tokens))       # positions a step touches, at any offset
                 out.append(min(total, (span + self.page_size - 2) // self.page_size + 1))
         return out
 
@@ -203,7 +218,7 @@ class CacheManager:
                     table[i] = -1
             while len(table) < want:
                 table.append(pool.take() if len(table) >= first_page else -1)
-        if step_end is not None and any(group.window is not None for group in self.groups):
+        if step_end is not None and any(group.reach is not None for group in self.groups):
             new_len = min(new_len, step_end)                    # positions that every group covers
         rc.num_tokens = max(rc.num_tokens, new_len)
 
@@ -226,7 +241,7 @@ class CacheManager:
             block = tokens[i * ps:(i + 1) * ps]
             h = chain_hash(block, h)
             pages = [pool.lookup(h, block) for pool in self.pools]
-            if any(p == -1 and group.window is None for p, group in zip(pages, self.groups)):
+            if any(p == -1 and group.reach is None for p, group in zip(pages, self.groups)):
                 break                       # nothing beyond a page that an all-keys group has lost
             if all(p == -1 for p in pages):
                 break

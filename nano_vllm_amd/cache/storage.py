@@ -20,8 +20,23 @@ from ..parts.model import LayerCache, torch_dtype
 
 def bytes_per_page(needs, groups, page_size: int, itemsize: int) -> List[int]:
     """Per group: bytes that one page takes over all the group's runs."""
-    return [sum(needs[r].num_kv_heads * (needs[r].head_dim + _value_dim(needs[r])) * page_size * itemsize
-                for r in g.runs) for g in groups]
+    return [sum(_paged(needs[r]).num_kv_heads * (_paged(needs[r]).head_dim + _value_dim(_paged(needs[r]))) * page_size
+                * itemsize for r in g.runs) for g in groups]
+
+
+def _paged(need):
+    """The keys-and-values part of a run's need (a need may combine pages and fixed state)."""
+    for part in getattr(need, "parts", (need,)):
+        if hasattr(part, "num_kv_heads"):
+            return part
+    return None
+
+
+def _fixed(need):
+    for part in getattr(need, "parts", (need,)):
+        if hasattr(part, "tensors"):
+            return part
+    return None
 
 
 def _value_dim(need) -> int:
@@ -32,7 +47,7 @@ def _value_dim(need) -> int:
 def state_bytes_per_slot(needs, state_runs) -> int:
     total = 0
     for r in state_runs:
-        for shape, dtype in needs[r].tensors.values():
+        for shape, dtype in _fixed(needs[r]).tensors.values():
             n = 1
             for s in shape:
                 n *= s
@@ -49,14 +64,15 @@ def allocate(needs, groups, state_runs, num_pages: Sequence[int], page_size: int
     caches: List[LayerCache] = [LayerCache() for _ in needs]
     for g, group in enumerate(groups):
         for r in group.runs:
-            need = needs[r]
+            need = _paged(needs[r])
             k = torch.zeros((num_pages[g], need.num_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
             v = torch.zeros(v_cache_shape(num_pages[g], need.num_kv_heads, _value_dim(need), page_size), dtype=dtype,
                             device=device)
             caches[r] = LayerCache(group=g, k=k, v=v)
     for r in state_runs:
-        caches[r] = LayerCache(state={
+        # (a run whose need combines pages and state keeps both in its one LayerCache)
+        caches[r].state = {
             # one row more than requests can hold: the slot of the rows that pad a captured batch
             name: torch.zeros((num_slots + 1,) + tuple(shape), dtype=_state_dtype(dt), device=device)
-            for name, (shape, dt) in needs[r].tensors.items()})
+            for name, (shape, dt) in _fixed(needs[r]).tensors.items()}
     return caches

@@ -1,8 +1,10 @@
-from .model_config import ConfigError, NozuraxConfig, NozuraxLayer, Qwen3Config, canonical_dtype, read_config_json
+from .model_config import (ChunkAttentionConfig, ConfigError, ExpertsConfig, MafaraxConfig, MafaraxLayer, NozuraxConfig,
+                           NozuraxLayer, Qwen3Config, StateSpaceConfig, canonical_dtype, read_config_json)
 from .engine_config import EngineConfig
 from .registry import (Architecture, register_architecture, get_architecture,
                        architecture_of, known_architectures)
 
-__all__ = ["ConfigError", "Qwen3Config", "NozuraxConfig", "NozuraxLayer", "canonical_dtype", "read_config_json", "EngineConfig",
+__all__ = ["ConfigError", "Qwen3Config", "NozuraxConfig", "NozuraxLayer", "MafaraxConfig", "MafaraxLayer",
+           "ChunkAttentionConfig", "StateSpaceConfig", "ExpertsConfig", "canonical_dtype", "read_config_json", "EngineConfig",
            "Architecture", "register_architecture", "get_architecture", "architecture_of",
            "known_architectures"]

@@ -322,3 +322,185 @@ class NozuraxConfig:
         if self.eos_token_id is not None:
             out["eos_token_id"] = list(self.eos_token_id)
         return out
+
+
+# ---------------------------------------------------------------------------- Mafarax
+def _whole(d: Mapping[str, Any], key: str, where: str, default=None) -> int:
+    """A positive whole number (config files may write 4 as 4.0)."""
+    v = d.get(key, default)
+    if v is None or isinstance(v, bool) or not isinstance(v, (int, float)) or v != int(v) or int(v) <= 0:
+        raise ConfigError(f"{where}: key {key!r} must be a positive whole number, got {v!r}")
+    return int(v)
+
+
+@dataclass(frozen=True)
+class ChunkAttentionConfig:
+    """The attention half of a side-by-side mixer: grouped keys and values, values of a size of their
+    own, biases, rotation of the first rot_dims channels of a head with every frequency divided by
+    rot_factor, a scale of its own, and a mask that lets a query read its own chunk of `chunk`
+    positions only.  rot_dims 0: no rotation."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    chunk: int
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_factor: float = 1.0
+
+
+@dataclass(frozen=True)
+class StateSpaceConfig:
+    """The state-space half: heads of vdim channels, a state of `state` rows per head, B and C shared
+    by the heads of a group, a causal convolution of `conv` taps, a gated norm in norm_groups parts."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int
+
+
+@dataclass(frozen=True)
+class ExpertsConfig:
+    """A routed feed-forward: `experts` experts of inner size ff, `top` per token, chosen among the
+    `keep` best of `group_count` groups of neighbouring experts; weights are the sigmoid scores
+    times `scale`; shared_ff: the inner size of the expert every token runs (None: no such expert)."""
+    experts: int
+    top: int
+    ff: int
+    scale: float
+    group_count: int = 1
+    group_keep: int = 1
+    shared_ff: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class MafaraxLayer:
+    left: ChunkAttentionConfig
+    right: StateSpaceConfig
+    mlp: Optional[ExpertsConfig]
+
+
+@dataclass(frozen=True)
+class MafaraxConfig:
+    """Mafarax: pre-norm layers on a float32 residual stream with Dynamic Tanh norms; every mixer is a
+    chunked attention and a state-space layer side by side on the same input, their outputs normed
+    and averaged; the feed-forward is a mixture of experts with a shared expert, or absent.
+    config.json gives every size and constant, layer by layer."""
+    vocab: int
+    width: int
+    eps: float
+    logit_scale: float
+    layers: Tuple[MafaraxLayer, ...]
+    dtype: str = "bfloat16"
+    eos_token_id: Optional[Tuple[int, ...]] = None
+    architecture: str = "Mafarax"
+
+    @classmethod
+    def from_dict(cls, d: Mapping[str, Any]) -> "MafaraxConfig":
+        where = "config.json"
+        entries = d.get("layers")
+        if not isinstance(entries, (list, tuple)) or not entries:
+            raise ConfigError(f"{where}: key 'layers' must be a list of layers")
+        layers = []
+        for i, entry in enumerate(entries):
+            at = f"{where}: layers[{i}]"
+            if not isinstance(entry, Mapping):
+                raise ConfigError(f"{at} must be an object")
+            if entry.get("type") != "parallel":
+                raise ConfigError(f"{at}: type must be 'parallel', got {entry.get('type')!r}")
+            mixer = _section(entry, "mixer", at)
+            l, r = _section(mixer, "left", at + ".mixer"), _section(mixer, "right", at + ".mixer")
+            la, ra = at + ".mixer.left", at + ".mixer.right"
+            rot = l.get("rot")
+            dims, base, factor = 0, 10000.0, 1.0
+            if rot is not None:
+                dims = _whole(rot, "dims", la + ".rot")
+                base = _require(rot, "base", float, la + ".rot")
+                scaling = rot.get("scaling")
+                if scaling is not None:
+                    factor = _require(scaling, "factor", float, la + ".rot.scaling")
+            mask = _section(l, "mask", la)
+            left = ChunkAttentionConfig(
+                heads=_whole(l, "heads", la), kv_heads=_whole(l, "kv_heads", la), dim=_whole(l, "dim", la),
+                vdim=_whole(l, "vdim", la), scale=_require(l, "scale", float, la), chunk=_whole(mask, "size", la + ".mask"),
+                rot_dims=dims, rot_base=base, rot_factor=factor)
+            right = StateSpaceConfig(
+                heads=_whole(r, "heads", ra), vdim=_whole(r, "vdim", ra), state=_whole(r, "state", ra),
+                groups=_whole(r, "groups", ra, 1), conv=_whole(r, "conv", ra),
+                norm_groups=_whole(r, "norm_groups", ra, 1))
+            mlp = entry.get("mlp")
+            experts = None
+            if mlp is not None:
+                ma = at + ".mlp"
+                if not isinstance(mlp, Mapping) or mlp.get("kind") != "moe":
+                    raise ConfigError(f"{ma} must be null or an object of kind 'moe', got {mlp!r}")
+                router = _section(mlp, "router", ma)
+                groups = router.get("groups")
+                shared = mlp.get("shared")
+                experts = ExpertsConfig(
+                    experts=_whole(router, "experts", ma + ".router"), top=_whole(router, "top", ma + ".router"),
+                    ff=_whole(_section(mlp, "expert", ma), "ff", ma + ".expert"),
+                    scale=float(router["scale"]) if router.get("scale") is not None else 1.0,
+                    group_count=1 if groups is None else _whole(groups, "count", ma + ".router.groups"),
+                    group_keep=1 if groups is None else _whole(groups, "keep", ma + ".router.groups"),
+                    shared_ff=None if shared is None else _whole(shared, "ff", ma + ".shared"))
+            layers.append(MafaraxLayer(left, right, experts))
+        norm = _section(d, "norm", where)
+        eos = d.get("eos_token_id")
+        eos = (eos,) if isinstance(eos, int) else tuple(int(x) for x in eos) if isinstance(eos, (list, tuple)) else None
+        cfg = cls(vocab=_whole(d, "vocab", where), width=_whole(d, "width", where),
+                  eps=_require(norm, "eps", float, where + ": norm"),
+                  logit_scale=float(d["logit_scale"]) if d.get("logit_scale") is not None else 1.0,
+                  layers=tuple(layers), dtype=canonical_dtype(d.get("dtype") or d.get("torch_dtype") or "bfloat16"),
+                  eos_token_id=eos, architecture=d.get("architecture") or (d.get("architectures") or ["Mafarax"])[0])
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if not (self.eps > 0):
+            raise ConfigError(f"config.json: norm.eps must be positive, got {self.eps}")
+        for i, layer in enumerate(self.layers):
+            at = f"config.json: layers[{i}]"
+            l, r, m = layer.left, layer.right, layer.mlp
+            if l.heads % l.kv_heads:
+                raise ConfigError(f"{at}: {l.heads} heads do not divide into {l.kv_heads} kv_heads")
+            if l.rot_dims % 2 or l.rot_dims > l.dim or (l.rot_dims and not (l.rot_base > 0 and l.rot_factor > 0)):
+                raise ConfigError(f"{at}: rot.dims {l.rot_dims} must be even and at most dim {l.dim}, rot.base and "
+                                  f"the scaling factor positive")
+            if r.heads % r.groups:
+                raise ConfigError(f"{at}: {r.heads} state-space heads do not divide into {r.groups} groups")
+            if (r.heads * r.vdim) % r.norm_groups:
+                raise ConfigError(f"{at}: {r.heads * r.vdim} inner channels do not divide into {r.norm_groups} norm groups")
+            if m is not None:
+                if m.experts % m.group_count or not 1 <= m.group_keep <= m.group_count:
+                    raise ConfigError(f"{at}: {m.experts} experts in {m.group_count} groups, of which {m.group_keep} are kept")
+                if m.top > m.group_keep * (m.experts // m.group_count):
+                    raise ConfigError(f"{at}: {m.top} experts a token cannot be chosen from {m.group_keep} groups of "
+                                      f"{m.experts // m.group_count}")
+
+    def to_dict(self) -> dict:
+        """The config.json that describes this configuration."""
+        entries = []
+        for layer in self.layers:
+            l, r, m = layer.left, layer.right, layer.mlp
+            left = {"heads": l.heads, "kv_heads": l.kv_heads, "dim": l.dim, "vdim": l.vdim, "scale": l.scale,
+                    "mask": {"size": l.chunk}}
+            if l.rot_dims:
+                left["rot"] = {"dims": l.rot_dims, "base": l.rot_base, "scaling": {"factor": l.rot_factor}}
+            right = {"heads": r.heads, "vdim": r.vdim, "state": r.state, "groups": r.groups, "conv": r.conv,
+                     "norm_groups": r.norm_groups}
+            mlp = None
+            if m is not None:
+                mlp = {"kind": "moe", "expert": {"ff": m.ff},
+                       "router": {"experts": m.experts, "top": m.top, "scale": m.scale,
+                                  "groups": {"count": m.group_count, "keep": m.group_keep}},
+                       "shared": None if m.shared_ff is None else {"ff": m.shared_ff}}
+            entries.append({"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp})
+        out = {"architecture": self.architecture, "vocab": self.vocab, "width": self.width, "norm": {"eps": self.eps},
+               "logit_scale": self.logit_scale, "layers": entries, "torch_dtype": self.dtype}
+        if self.eos_token_id is not None:
+            out["eos_token_id"] = list(self.eos_token_id)
+        return out

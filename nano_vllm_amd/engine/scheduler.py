@@ -61,7 +61,7 @@ class Scheduler:
         # with every token; what happens when it runs out is the scheduler's business, see above.)
         final = min(seq.num_tokens + seq.max_tokens, self.max_model_len)
         for g, pages in enumerate(self.cache.peak_pages(final, 1)):
-            if self.cache.groups[g].window is not None:
+            if self.cache.groups[g].reach is not None:
                 need[g] = max(need[g], pages)
         for g, (pages, pool) in enumerate(zip(need, self.cache.pools)):
             if pages > pool.num_pages:

@@ -15,6 +15,13 @@ Options beyond the reference's attention, each a parameter:
     q_temperature (coef, every)     q *= 1 + coef * ln(floor((p + 1) / every) + 1) at position p
     sink                            a learned number per head whose exponential joins the softmax's
                                     denominator: a key without a value that every query sees once
+    chunk                           a query at position p reads the keys of positions floor(p / chunk) *
+                                    chunk ... p only: the sequence is cut into chunks counted from its
+                                    position 0, wherever a prompt was cut for processing
+    o_bias                          a bias on the output projection
+With values of their own size (or whole-projection norms, or a temperature) the position encoding's
+rotation is applied by the same preparation kernel, from the cosines and sines of the step's tokens
+(position_encoding.step_table): such a model needs no table of all positions.
 
 Interface of a mixer:
     cache_need()                 -> PagedKV | FixedState | None
@@ -36,7 +43,8 @@ class Attention(Part):
     keys), scale (None: head_dim^-0.5), reads_shared_cache (bool: the run owns no cache, it
     projects q only and reads another run's keys and values), v_head_dim (None: head_dim),
     qk_norm_scope ("head" | "projection"), q_temperature (None or {"coef", "every"}), sink (bool),
-    and the names of the checkpoint tensors (q_name, ..., q_norm_name, k_norm_name, sink_name)."""
+    chunk (None or positions), o_bias (bool), step_rotation (bool: rotate from the step's own table
+    also where the per-head kernel could serve), and the names of the checkpoint tensors (q_name, ..., q_norm_name, k_norm_name, sink_name)."""
 
     def __init__(self, params: Mapping, build: BuildContext):
         super().__init__(params, build)
@@ -51,6 +59,10 @@ class Attention(Part):
         self.eps = float(p.get("eps", 1e-6))
         self.bias = bool(p.get("bias", False))
         self.window = p.get("window")
+        self.chunk = p.get("chunk")
+        if self.chunk is not None and int(self.chunk) <= 0:
+            raise ValueError(f"attention: a chunk of {self.chunk} positions")
+        self.o_bias = bool(p.get("o_bias", False))
         scale = p.get("scale")
         self.scale = float(scale) if scale is not None else self.head_dim ** -0.5     # qwen3.py:39
         self.shared = bool(p.get("reads_shared_cache", False))
@@ -72,10 +84,11 @@ class Attention(Part):
         self.sink = bool(p.get("sink", False))
         # The whole-projection preparation has its own kernel, which also scales q by its temperature
         # and stores values of their own size; the per-head one rotates.  Each does what its model needs.
-        self.row_prepare = self.norm_scope == "projection" or self.temp_coef != 0.0 or self.v_head_dim != self.head_dim
-        if self.row_prepare and self.position_encoding is not None:
-            raise ValueError("attention: a position encoding goes with per-head norms, equal head sizes and no "
-                             "query temperature")
+        self.row_prepare = self.norm_scope == "projection" or self.temp_coef != 0.0 or self.v_head_dim != self.head_dim \
+            or bool(p.get("step_rotation", False))
+        if self.row_prepare and self.position_encoding is not None and not hasattr(self.position_encoding, "step_table"):
+            raise ValueError("attention: with whole-projection norms, a query temperature or values of their own "
+                             "size the position encoding must offer step_table")
         if self.row_prepare and self.qk_norm and self.norm_scope == "head":
             raise ValueError("attention: per-head norms go with equal head sizes and no query temperature")
 
@@ -83,8 +96,9 @@ class Attention(Part):
     def kernel_modules(self):
         prepare = "qk_rownorm" if self.row_prepare else "rope"
         if self.v_head_dim != self.head_dim:
-            return (prepare, "attn_generic")
-        return (prepare, "attn_generic", "attn_decode", "attn_prefill")
+            return (prepare, "attn_generic") + (("rope",) if self.row_prepare and self.position_encoding else ())
+        return (prepare, "attn_generic", "attn_decode", "attn_prefill") + \
+            (("rope",) if self.row_prepare and self.position_encoding else ())
 
     # ------------------------------------------------------------------ declaration
     def param_decls(self) -> Dict[str, ParamDecl]:
@@ -111,13 +125,16 @@ class Attention(Part):
         if self.sink:
             d["sinks"] = ParamDecl((self.heads,), dtype="float32", sources=(Source(self.sink_name, 0, self.heads),))
         d[f"{self.o_name}.weight"] = ParamDecl((h, self.heads * self.v_head_dim))
+        if self.o_bias:
+            d[f"{self.o_name}.bias"] = ParamDecl((h,))
         return d
 
     def cache_need(self):
         if self.shared:
             return None
         return PagedKV(self.kv_heads, self.head_dim, self.window,
-                       None if self.v_head_dim == self.head_dim else self.v_head_dim)
+                       None if self.v_head_dim == self.head_dim else self.v_head_dim,
+                       None if self.chunk is None else int(self.chunk))
 
     # ------------------------------------------------------------------ forward
     def forward(self, x, batch, cache):
@@ -126,7 +143,7 @@ class Attention(Part):
         kv_heads = 0 if self.shared else self.kv_heads
         # deferred: the products below are handed to the q/k preparation and to the block's norm only
         pe = self.position_encoding
-        table = pe.rotary_table() if pe is not None else None
+        table = pe.rotary_table() if pe is not None and not self.row_prepare else None
         qkv = k.linear(x, w["qkv_proj.weight"], w.get("qkv_proj.bias"),
                        deferred=self.row_prepare or pe is None or table is not None)
         group = batch.groups[cache.group]
@@ -135,8 +152,9 @@ class Attention(Part):
         qw = w.get("q_norm.weight")
         kw = w.get("k_norm.weight")
         if self.row_prepare:
+            extra = {"rot_table": pe.step_table(batch)} if pe is not None else {}
             q = k.qk_rownorm_store(qkv, self.heads, kv_heads, self.head_dim, self.v_head_dim, qw, kw, self.eps,
-                                   batch.positions, self.temp_coef, self.temp_every, slots, kc, vc)
+                                   batch.positions, self.temp_coef, self.temp_every, slots, kc, vc, **extra)
         elif pe is None or table is not None:
             q = k.qk_norm_rope_store(qkv, self.heads, kv_heads, self.head_dim, qw, kw, self.eps, table,
                                      batch.positions, slots, kc, vc, max_position=batch.max_kv_len)
@@ -150,13 +168,14 @@ class Attention(Part):
             if not self.shared:
                 k.qk_norm_rope_store(qkv, self.heads, kv_heads, self.head_dim, None, None, self.eps, None, None,
                                      slots, kc, vc)
+        extra = {"chunk": int(self.chunk)} if self.chunk is not None else {}
         if self.sink or self.v_head_dim != self.head_dim:
             o = k.paged_attention(q, self.heads, self.kv_heads, self.head_dim, cache.k, cache.v, batch, cache.group,
-                                  self.scale, self.window, v_head_dim=self.v_head_dim, sinks=w.get("sinks"))
+                                  self.scale, self.window, v_head_dim=self.v_head_dim, sinks=w.get("sinks"), **extra)
         else:
             o = k.paged_attention(q, self.heads, self.kv_heads, self.head_dim, cache.k, cache.v, batch, cache.group,
-                                  self.scale, self.window)
-        return k.linear(o, w[f"{self.o_name}.weight"], deferred=True)
+                                  self.scale, self.window, **extra)
+        return k.linear(o, w[f"{self.o_name}.weight"], w.get(f"{self.o_name}.bias"), deferred=True)
 
 
 register_part("mixer", "attention", Attention)

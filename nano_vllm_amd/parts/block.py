@@ -6,6 +6,10 @@ next norm (nanovllm/models/qwen3.py:146-159):
     later layers: r = h + r;       x = norm1(r)
     a = mixer(x);  r = a + r;  y = norm2(r);  m = feed_forward(y);  returns (m, r)
 The caller adds the last m to r inside the final norm (qwen3.py:182).
+With the parameter stream = "float32" the residual stream r is kept in float32 whatever the element
+type: every sublayer's output travels as a list of one addend, which the next norm adds to the stream
+(the norms of such a block take lists: rms_norm and dynamic_tanh do), and the layer may have no
+feed-forward (then it has no second norm either).
 
 "parallel_residual": one norm whose output both sublayers read, their sum added to the stream:
     x = norm(r);  r <- r + (mixer(x) + feed_forward(x))
@@ -32,14 +36,21 @@ class PreNormResidualBlock(Part):
         super().__init__(params, build)
         parts = params["parts"]            # role -> PartSpec
         names = params["names"]            # role -> name in checkpoint tensor names
-        missing = [r for r in self.ROLES if r not in parts]
+        stream = params.get("stream")
+        if stream not in (None, "float32"):
+            raise ValueError(f"pre_norm_residual block: stream must be 'float32' or absent, got {stream!r}")
+        self.float_stream = stream == "float32"
+        optional = ("feed_forward_norm", "feed_forward") if self.float_stream and not parts.get("feed_forward") else ()
+        missing = [r for r in self.ROLES if r not in parts and r not in optional]
         if missing:
             raise ValueError(f"pre_norm_residual block: missing parts {missing}")
         self.mixer_norm = make_part("norm", parts["mixer_norm"], build)
         self.mixer = make_part("mixer", parts["mixer"], build)
-        self.feed_forward_norm = make_part("norm", parts["feed_forward_norm"], build)
-        self.feed_forward = make_part("feed_forward", parts["feed_forward"], build)
-        self._children = {names[r]: getattr(self, r) for r in self.ROLES}
+        self.feed_forward_norm = self.feed_forward = None
+        if parts.get("feed_forward"):
+            self.feed_forward_norm = make_part("norm", parts["feed_forward_norm"], build)
+            self.feed_forward = make_part("feed_forward", parts["feed_forward"], build)
+        self._children = {names[r]: getattr(self, r) for r in self.ROLES if getattr(self, r) is not None}
 
     def children(self) -> Dict[str, Part]:
         return self._children
@@ -52,6 +63,14 @@ class PreNormResidualBlock(Part):
         return self.mixer.replays_state_steps
 
     def forward(self, h, residual, batch, cache):
+        if self.float_stream:
+            addends = tuple(h) if isinstance(h, (tuple, list)) else (h,)
+            x, residual = self.mixer_norm.forward_add(addends, residual)
+            a = self.mixer.forward(x, batch, cache)
+            if self.feed_forward is None:
+                return (a,), residual
+            y, residual = self.feed_forward_norm.forward_add((a,), residual)
+            return (self.feed_forward.forward(y, batch),), residual
         if residual is None:
             x, residual = self.mixer_norm.forward(h), h
         else:

@@ -30,18 +30,23 @@ class TokenEmbedding(Part):
 
 class OutputHead(Part):
     """logits = x W^T in float32, W [vocab, hidden] (embed_head.py:61); tied: W is the
-    embedding's storage and the checkpoint holds no tensor for it (qwen3.py:202-203)."""
+    embedding's storage and the checkpoint holds no tensor for it (qwen3.py:202-203).  With the
+    parameter logit_scale the logits are multiplied by that constant, in float."""
 
     def __init__(self, params: Mapping, build: BuildContext):
         super().__init__(params, build)
         self.vocab, self.hidden = int(params["vocab_size"]), int(params["hidden_size"])
         self.tied = bool(params.get("tied", False))
+        self.logit_scale = float(params.get("logit_scale", 1.0))
 
     def param_decls(self):
         return {} if self.tied else {"weight": ParamDecl((self.vocab, self.hidden))}
 
     def forward(self, x):
-        return self.kernels.linear(x, self.weights["weight"], out_float32=True)
+        logits = self.kernels.linear(x, self.weights["weight"], out_float32=True)
+        if self.logit_scale != 1.0:
+            self.kernels.scale_(logits, self.logit_scale)
+        return logits
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)

@@ -1,0 +1,102 @@
+"""Feed-forward parts without a gate, and a mixture of them.
+
+"mlp": m = act(y Wu^T) Wd^T, act one of relu2 (the square of relu), relu, silu, gelu_tanh.
+
+"moe": every token runs `top` of `experts` such layers (no biases) and, optionally, a shared one:
+    s = sigmoid(y Wr^T)                       router scores, float
+    experts form group_count equal groups of neighbours; a group's score is the sum of its two largest
+    scores (of its one score where groups hold one expert); only experts of the group_keep best groups
+    can be chosen; of those the `top` with the largest scores are
+    m = sum over the chosen e of (scale * s_e) expert_e(y)  +  shared(y)
+The weights are the scores themselves, not renormalised.  Routing is decided on the device and the
+experts' products run over the tokens sorted by expert, so a step never asks the host how many
+tokens an expert got: the same launches whatever the routing.
+"""
+from __future__ import annotations
+
+from typing import Dict, Mapping
+
+from .base import BuildContext, ParamDecl, Part, Source
+from .registry import make_part, register_part
+
+ACTIVATIONS = ("relu2", "relu", "silu", "gelu_tanh")
+
+
+class PlainMLP(Part):
+    """params: hidden_size, intermediate_size, activation (default relu2), up_name, down_name."""
+
+    def __init__(self, params: Mapping, build: BuildContext):
+        super().__init__(params, build)
+        self.hidden = int(params["hidden_size"])
+        self.inner = int(params["intermediate_size"])
+        self.up_name = params.get("up_name", "up_proj")
+        self.down_name = params.get("down_name", "down_proj")
+        self.activation = params.get("activation", "relu2")
+        if self.activation not in ACTIVATIONS:
+            raise ValueError(f"mlp: unknown activation {self.activation!r}")
+
+    def param_decls(self) -> Dict[str, ParamDecl]:
+        return {f"{self.up_name}.weight": ParamDecl((self.inner, self.hidden)),
+                f"{self.down_name}.weight": ParamDecl((self.hidden, self.inner))}
+
+    def forward(self, x, batch=None):
+        z = self.kernels.act(self.kernels.linear(x, self.weights[f"{self.up_name}.weight"]), self.activation)
+        return self.kernels.linear(z, self.weights[f"{self.down_name}.weight"], deferred=True)
+
+
+class MixtureOfExperts(Part):
+    """params: hidden_size, num_experts, top, intermediate_size, scale, group_count, group_keep,
+    activation, shared (a PartSpec of a feed-forward, or None), and names: router_name, shared_name,
+    expert_name (a format with {} for the expert's number), up_name, down_name."""
+
+    kernel_modules = ("moe",)
+
+    def __init__(self, params: Mapping, build: BuildContext):
+        super().__init__(params, build)
+        p = params
+        self.hidden = int(p["hidden_size"])
+        self.experts = int(p["num_experts"])
+        self.top = int(p["top"])
+        self.inner = int(p["intermediate_size"])
+        self.scale = float(p.get("scale", 1.0))
+        self.group_count = int(p.get("group_count", 1))
+        self.group_keep = int(p.get("group_keep", self.group_count))
+        self.activation = p.get("activation", "relu2")
+        if self.activation not in ACTIVATIONS:
+            raise ValueError(f"moe: unknown activation {self.activation!r}")
+        if self.experts % self.group_count or not 1 <= self.group_keep <= self.group_count:
+            raise ValueError(f"moe: {self.experts} experts in {self.group_count} groups of which {self.group_keep} are kept")
+        if not 1 <= self.top <= self.group_keep * (self.experts // self.group_count):
+            raise ValueError(f"moe: {self.top} experts a token out of {self.group_keep} groups of "
+                             f"{self.experts // self.group_count}")
+        self.router_name = p.get("router_name", "router")
+        self.shared_name = p.get("shared_name", "shared")
+        self.expert_name = p.get("expert_name", "experts.{}")
+        self.up_name, self.down_name = p.get("up_name", "up_proj"), p.get("down_name", "down_proj")
+        self.shared = make_part("feed_forward", p["shared"], build) if p.get("shared") else None
+
+    def children(self) -> Dict[str, Part]:
+        return {self.shared_name: self.shared} if self.shared is not None else {}
+
+    def param_decls(self) -> Dict[str, ParamDecl]:
+        e, i, h = self.experts, self.inner, self.hidden
+        name = self.expert_name.format
+        return {
+            f"{self.router_name}.weight": ParamDecl((e, h)),
+            # the experts' matrices one below the other: expert n's rows are [n * rows, (n + 1) * rows)
+            "up.weight": ParamDecl((e * i, h), sources=tuple(
+                Source(f"{name(n)}.{self.up_name}.weight", n * i, i) for n in range(e))),
+            "down.weight": ParamDecl((e * h, i), sources=tuple(
+                Source(f"{name(n)}.{self.down_name}.weight", n * h, h) for n in range(e))),
+        }
+
+    def forward(self, x, batch=None):
+        k, w = self.kernels, self.weights
+        logits = k.linear(x, w[f"{self.router_name}.weight"], out_float32=True)
+        ids, weights = k.moe_route(logits, self.top, self.group_count, self.group_keep, self.scale)
+        shared = self.shared.forward(x, batch) if self.shared is not None else None
+        return k.moe_experts(x, ids, weights, w["up.weight"], w["down.weight"], self.experts, self.activation, add=shared)
+
+
+register_part("feed_forward", "mlp", PlainMLP)
+register_part("feed_forward", "moe", MixtureOfExperts)

@@ -7,6 +7,10 @@ With weight_offset c the factor is (c + weight): c = 1 is the weight stored arou
 with an offset, and every norm that is handed a list of addends instead of one tensor, works on a
 residual stream kept in float32: the stream takes the sum of the addends, the norm is computed in
 float and rounded once to the element type.
+
+"dynamic_tanh": y = tanh(alpha * x) * weight + bias with one learned number alpha per norm: no mean,
+no variance, every entry by itself.  It works on a float32 residual stream (a list of addends, as
+above); tanh, products and sums in float, rounded once.
 """
 from __future__ import annotations
 
@@ -45,4 +49,30 @@ class RMSNorm(Part):
         return self.kernels.add_rms_norm(x, residual, self.weights["weight"], self.eps, out=out)
 
 
+class DynamicTanh(Part):
+    """params: dim; optional names of the checkpoint tensors below the norm's own (bias_name, alpha_name)."""
+
+    def __init__(self, params: Mapping, build: BuildContext):
+        super().__init__(params, build)
+        self.dim = int(params["dim"])
+        self.bias_name = params.get("bias_name", "bias")
+        self.alpha_name = params.get("alpha_name", "alpha")
+
+    def param_decls(self) -> Dict[str, ParamDecl]:
+        return {"weight": ParamDecl((self.dim,), dtype="float32", init="norm"),
+                self.bias_name: ParamDecl((self.dim,), dtype="float32"),
+                self.alpha_name: ParamDecl((), dtype="float32", init="norm")}
+
+    def forward(self, x, out=None):
+        return self.forward_add((x,), None, out=out)[0]
+
+    def forward_add(self, x, residual, out=None):
+        """residual <- residual + sum of the addends x (None: the stream starts as their sum);
+        returns (tanh(alpha * residual) * weight + bias, residual)."""
+        addends = tuple(x) if isinstance(x, (tuple, list)) else (x,)
+        w = self.weights
+        return self.kernels.stream_dyt(addends, residual, w["weight"], w[self.bias_name], w[self.alpha_name], out=out)
+
+
 register_part("norm", "rms_norm", RMSNorm)
+register_part("norm", "dynamic_tanh", DynamicTanh)

@@ -13,6 +13,11 @@ angle = position * inv_freq_i in float32 whatever the model's element type, pair
 The reference rotates the whole head (qwen3.py:49-54 passes rotary_dim = head_dim); with a
 smaller rotary_dim R the table is R wide and the first R channels of a head are rotated, in
 pairs (i, i + R/2), the others left as they are.
+With scaling_factor every frequency is divided by that constant (positions stretched linearly).
+A mixer whose model names no longest sequence asks for step_table(batch) instead of the table of all
+positions: the cosines and sines of the step's own tokens, [tokens, R], made once per step by a
+kernel that reads the positions on the device (so a captured step makes it anew at every replay) and
+shared by all the layers that rotate alike.
 "none": no encoding.
 """
 from __future__ import annotations
@@ -27,7 +32,7 @@ from .registry import register_part
 
 class RotaryNeox(Part):
     """params: head_dim, theta, max_position (rows of the table), rotary_dim (channels of a head
-    that are rotated; default all)."""
+    that are rotated; default all), scaling_factor (default 1)."""
 
     def __init__(self, params: Mapping, build: BuildContext):
         super().__init__(params, build)
@@ -42,9 +47,27 @@ class RotaryNeox(Part):
         # The reference's own float32 expression (rotary_embedding.py:29), evaluated on the host:
         # the angles' rounding is part of the model.
         inv_freq = 1.0 / (self.theta ** (torch.arange(0, self.rotary_dim, 2, dtype=torch.float) / self.rotary_dim))
+        self.scaling_factor = float(params.get("scaling_factor", 1.0))
+        if not self.scaling_factor > 0:
+            raise ValueError(f"rotary_neox: the scaling factor must be positive, got {self.scaling_factor}")
+        if self.scaling_factor != 1.0:
+            inv_freq = inv_freq / self.scaling_factor
         self.inv_freq = inv_freq
         self._device = build.device
         self._table = None
+        self._inv_freq_dev = None
+
+    def step_table(self, batch) -> torch.Tensor:
+        """float32 [tokens, rotary_dim]: cosines, then sines, of the step's tokens at their positions."""
+        kept = getattr(batch, "step_cache", None)
+        if kept is None:
+            kept = batch.step_cache = {}
+        key = ("rotary_step", self.rotary_dim, self.theta, self.scaling_factor)
+        if key not in kept:
+            if self._inv_freq_dev is None:
+                self._inv_freq_dev = self.inv_freq.to(self._device)
+            kept[key] = self.kernels.rotary_step_table(self._inv_freq_dev, batch.positions)
+        return kept[key]
 
     def rotary_table(self) -> Optional[torch.Tensor]:
         if self._table is None:            # made on first use: building a part touches no device

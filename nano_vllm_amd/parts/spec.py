@@ -93,11 +93,15 @@ class ModelSpec:
 class PagedKV:
     """Keys and values of every token, in pages.  window None: all keys stay; an integer:
     a query at position p reads positions > p - window only, and pages wholly before that
-    are given back.  v_head_dim: the size of a head's values where it is not head_dim."""
+    are given back.  chunk: a query at position p reads positions >= floor(p / chunk) * chunk only
+    (the sequence is cut into chunks counted from its position 0, and no query looks out of its
+    own); pages wholly before the chunk of the next query are given back.  v_head_dim: the size of
+    a head's values where it is not head_dim."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     v_head_dim: Optional[int] = None
+    chunk: Optional[int] = None
 
     @property
     def value_dim(self) -> int:
@@ -108,3 +112,33 @@ class PagedKV:
 class FixedState:
     """State of fixed size per request, kept in a slot: name -> (shape, dtype name)."""
     tensors: Mapping[str, Tuple[Tuple[int, ...], str]]
+
+
+@dataclass(frozen=True)
+class CombinedNeed:
+    """What a run needs whose mixer is made of several: each part's need, in the parts' order.  At
+    most one of them may be paged keys and values and at most one fixed state (the run's LayerCache
+    has one place for each)."""
+    parts: Tuple[Any, ...]
+
+    def __post_init__(self):
+        paged = [p for p in self.parts if isinstance(p, PagedKV)]
+        fixed = [p for p in self.parts if isinstance(p, FixedState)]
+        if len(paged) > 1 or len(fixed) > 1 or len(paged) + len(fixed) != len(self.parts):
+            raise ValueError("a combined cache need holds at most one PagedKV and one FixedState")
+
+
+def paged_need(need):
+    """The PagedKV of a need (its own, or the one inside a combined need), else None."""
+    for part in getattr(need, "parts", (need,)):
+        if hasattr(part, "num_kv_heads"):
+            return part
+    return None
+
+
+def state_need(need):
+    """The FixedState of a need (its own, or the one inside a combined need), else None."""
+    for part in getattr(need, "parts", (need,)):
+        if hasattr(part, "tensors"):
+            return part
+    return None

@@ -87,6 +87,86 @@ class TorchKernels:
             return out, residual
         return y, residual
 
+    def stream_dyt(self, addends, residual, weight, bias, alpha, out=None):
+        """The float32 stream takes the sum of the addends; tanh(alpha * stream) * weight + bias, rounded once."""
+        add = None
+        for a in addends:
+            add = a.float() if add is None else add + a.float()
+        if residual is None:
+            residual = add.clone()
+        elif add is not None:
+            residual += add
+        dt = addends[0].dtype if addends else out.dtype
+        y = (torch.tanh(alpha.float() * residual) * weight.float() + bias.float()).to(dt)
+        if out is not None:
+            out.copy_(y)
+            return out, residual
+        return y, residual
+
+    def pair_norm_mean(self, a, wa, b, wb, eps, out=None):
+        """Half the sum of the two inputs, each normed over its row with its plain weight."""
+        def normed(x, w):
+            x = x.float()
+            return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        y = (0.5 * (normed(a, wa) + normed(b, wb))).to(a.dtype)
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
+
+    def scale_(self, x, factor):
+        return x.mul_(factor)
+
+    @staticmethod
+    def _activation(g, act):
+        if act == "relu2":
+            return torch.relu(g) ** 2
+        if act == "relu":
+            return torch.relu(g)
+        if act == "silu":
+            return g * torch.sigmoid(g)
+        if act == "gelu_tanh":
+            return 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))
+        raise ValueError(act)
+
+    def act(self, x, act="relu2", out=None):
+        y = self._activation(x.float(), act).to(x.dtype)
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
+
+    # routed feed-forward
+    def moe_route(self, logits, top, group_count, group_keep, scale):
+        """int32 [T, top] experts and float32 [T, top] weights (scale * sigmoid score) of every token."""
+        T, E = logits.shape
+        s = torch.sigmoid(logits.float())
+        per = E // group_count
+        grouped = s.view(T, group_count, per)
+        group_score = grouped.topk(min(2, per), dim=-1).values.sum(-1)
+        kept = group_score.topk(group_keep, dim=-1).indices
+        allowed = torch.zeros((T, group_count), dtype=torch.bool, device=logits.device)
+        allowed.scatter_(1, kept, True)
+        masked = grouped.masked_fill(~allowed[:, :, None], float("-inf")).view(T, E)
+        ids = masked.topk(top, dim=-1).indices
+        return ids.to(torch.int32), (s.gather(1, ids) * scale).float()
+
+    def moe_experts(self, x, ids, weights, up, down, num_experts, act="relu2", add=None):
+        """sum over a token's experts e of weight * act(x Wu_e^T) Wd_e^T (+ add); up [E * ff, K], down [E * K, ff]."""
+        T, K = x.shape
+        ff = up.shape[0] // num_experts
+        out = torch.zeros((T, K), dtype=torch.float32, device=x.device)
+        for e in range(num_experts):
+            hit = ids == e
+            rows = hit.any(-1)
+            if bool(rows.any()):
+                h = self._activation((x[rows].float() @ up[e * ff:(e + 1) * ff].float().T), act).to(x.dtype).float()
+                y = (h @ down[e * K:(e + 1) * K].float().T).to(x.dtype).float()
+                out[rows] += (weights * hit)[rows].sum(-1, keepdim=True) * y
+        if add is not None:
+            out += add.float()
+        return out.to(x.dtype)
+
     # feed-forward (activation.py:8-11)
     def act_mul(self, gate_up, act="silu", out=None):
         inner = gate_up.shape[1] // 2
@@ -168,24 +248,39 @@ class TorchKernels:
                 v_cache[page, :, off // vt, :, off % vt] = v[ok]
         return qkv[:, :qd]
 
+    def rotary_step_table(self, inv_freq, positions):
+        ang = positions.float()[:, None] * inv_freq[None, :]
+        return torch.cat((ang.cos(), ang.sin()), dim=-1)
+
     def qk_rownorm_store(self, qkv, num_heads, num_kv_heads, head_dim, v_head_dim, q_weight, k_weight, eps,
-                         positions, temp_coef, temp_every, slots, k_cache, v_cache):
-        """q and k normed over the whole projection, q times its position's temperature, k and v stored."""
+                         positions, temp_coef, temp_every, slots, k_cache, v_cache, rot_table=None):
+        """q and k normed over the whole projection, q times its position's temperature, both rotated by
+        the rows of rot_table (one per token: cosines, then sines, for the first channels of a head),
+        k and v stored."""
         T = qkv.shape[0]
         qd, kd = num_heads * head_dim, num_kv_heads * head_dim
         dt = qkv.dtype
+
+        def turn(x, heads):
+            if rot_table is None:
+                return x
+            R = rot_table.shape[1]
+            x = x.reshape(T, heads, head_dim)
+            cos, sin = rot_table[:, None, : R // 2], rot_table[:, None, R // 2:]
+            a, b = x[..., : R // 2], x[..., R // 2:R]
+            return torch.cat((a * cos - b * sin, b * cos + a * sin, x[..., R:]), dim=-1).reshape(T, heads * head_dim)
         q = qkv[:, :qd].float()
         if q_weight is not None:
             q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_weight.float()
         if temp_coef:
             steps = torch.div(positions.long() + 1, int(temp_every), rounding_mode="floor").float()
             q = q * (1.0 + temp_coef * torch.log(steps + 1.0))[:, None]
-        qkv[:, :qd] = q.to(dt)
+        qkv[:, :qd] = turn(q, num_heads).to(dt)
         if num_kv_heads:
             k = qkv[:, qd:qd + kd].float()
             if k_weight is not None:
                 k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_weight.float()
-            qkv[:, qd:qd + kd] = k.to(dt)
+            qkv[:, qd:qd + kd] = turn(k, num_kv_heads).to(dt)
             if k_cache is not None:
                 page_size, vt = k_cache.shape[2], v_cache.shape[4]
                 s = slots.long()
@@ -233,9 +328,50 @@ class TorchKernels:
             return out
         return y
 
+    def state_space(self, proj, heads, vdim, n_state, groups, taps, conv_w, conv_b, dt_bias, a_log, d_skip, norm_w,
+                    norm_groups, eps, conv_state, ssm_state, batch, out=None):
+        """Token by token: the convolution over the request's last inputs, the step size, the state's
+        decay and update, the read-out, the gate and the grouped norm."""
+        T = proj.shape[0]
+        inner, gn = heads * vdim, groups * n_state
+        C = inner + 2 * gn
+        p = proj.float()
+        z, xbc, dt_raw = p[:, :inner], p[:, inner:inner + C], p[:, inner + C:]
+        y = torch.zeros((T, inner), dtype=torch.float32, device=proj.device)
+        slots = batch.state_slots.tolist()
+        a = -torch.exp(a_log.float())
+        per = heads // groups
+        t = 0
+        for s, (start, n) in enumerate(zip(batch.starts, batch.q_lens)):
+            slot = slots[s]
+            hist = conv_state[slot].clone() if start > 0 else torch.zeros_like(conv_state[slot])      # [C, taps - 1]
+            S = ssm_state[slot].clone() if start > 0 else torch.zeros_like(ssm_state[slot])           # [heads, N, P]
+            for i in range(t, t + n):
+                window = torch.cat((hist, xbc[i][:, None]), dim=1)                                    # [C, taps]
+                c = (window * conv_w.float()).sum(-1) + conv_b.float()
+                c = (c * torch.sigmoid(c)).to(proj.dtype).float()
+                hist = window[:, 1:]
+                x = c[:inner].reshape(heads, vdim)
+                B = c[inner:inner + gn].reshape(groups, n_state).repeat_interleave(per, 0)
+                Cc = c[inner + gn:].reshape(groups, n_state).repeat_interleave(per, 0)
+                dt = torch.nn.functional.softplus(dt_raw[i] + dt_bias.float(), threshold=1e9)
+                S = torch.exp(a * dt)[:, None, None] * S + dt[:, None, None] * B[:, :, None] * x[:, None, :]
+                y[i] = (torch.einsum("hnp,hn->hp", S, Cc) + d_skip.float()[:, None] * x).reshape(inner)
+            conv_state[slot] = hist
+            ssm_state[slot] = S
+            t += n
+        y = y * (z * torch.sigmoid(z))
+        y = y.reshape(T, norm_groups, inner // norm_groups)
+        y = (y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, inner) * norm_w.float()
+        y = y.to(proj.dtype)
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
+
     # attention (attention.py:64-75): token by token through the block table
     def paged_attention(self, q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, batch, group, scale,
-                        window=None, out=None, v_head_dim=None, sinks=None):
+                        window=None, out=None, v_head_dim=None, sinks=None, chunk=None):
         T = q.shape[0]
         D, G = head_dim, num_heads // num_kv_heads
         DV = v_head_dim or head_dim
@@ -246,6 +382,8 @@ class TorchKernels:
         for t in range(T):
             pos, seq = pos_l[t], seq_l[t]
             first = max(0, pos - window + 1) if window else 0
+            if chunk:
+                first = max(first, pos // chunk * chunk)
             js = torch.arange(first, pos + 1, device=q.device)
             pages = tables[seq].long()[js // page_size]
             assert bool((pages >= 0).all()), "a visible key has no page"
