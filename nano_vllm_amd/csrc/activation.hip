@@ -81,4 +81,26 @@ NVA_EXPORT int NVA_NAME(nva_silu_mul)(const void* x, int64_t x_stride, void* out
     return launch_act_mul<NVA_ACT_SILU>(x, x_stride, out, out_stride, rows, inner, stream);
 }
 
+// An activation without a gate: out[t, i] = act(x[t, i]); act by the codes of nva_gate_act (3: relu squared).
+template <typename T>
+__global__ void __launch_bounds__(256)
+act_kernel(const T* __restrict__ x, int64_t x_stride, T* __restrict__ out, int64_t out_stride, int64_t rows, int width, int act) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * width) return;
+    const int64_t r = idx / width;
+    const int i = (int)(idx % width);
+    out[r * out_stride + i] = from_float<T>(nva_gate_act(act, to_float(x[r * x_stride + i])));
+}
+
+NVA_EXPORT int NVA_NAME(nva_act)(const void* x, int64_t x_stride, void* out, int64_t out_stride, int64_t rows, int width,
+                                 int act, hipStream_t stream) {
+    if (rows == 0) return 0;
+    if (rows < 0 || width <= 0 || act < 0 || act > 3) return nva_fail("act: bad shape rows=%lld width=%d or activation %d", (long long)rows, width, act);
+    const int64_t total = rows * width;
+    if ((total + 255) / 256 > 0x7fffffff) return nva_fail("act: too many entries");
+    hipLaunchKernelGGL((act_kernel<elem_t>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (const elem_t*)x,
+                       x_stride, (elem_t*)out, out_stride, rows, width, act);
+    return nva_check_launch("act");
+}
+
 NVA_DEFINE_LAST_ERROR(nva_activation)

@@ -7,7 +7,8 @@
 //
 // Semantics (nanovllm/layers/attention.py:64-75 with causal=True): the query of a token at
 // absolute position p of its request, head h, reads the keys of kv head h / (Hq / Hkv) at
-// positions j <= p (and j > p - window if window > 0) through the request's block table:
+// positions j <= p (and j > p - window if window > 0, and j >= floor(p / chunk) * chunk if chunk > 0:
+// a query reads its own chunk of positions only) through the request's block table:
 // s_j = scale * <q, k_j>, P = softmax(s), o = sum_j P_j v_j.  The step's own keys are in the
 // cache already when this runs.
 // Layouts: K [pages, Hkv, page, D], V transposed in tiles of keys (common.h).  One wave per (token, q head).
@@ -18,7 +19,9 @@
 // Portions of prompts have a second kernel with the same arithmetic, operation for operation (the
 // results are the same bits): a workgroup takes 32 query rows of one request and one head, and the
 // chunks of 64 keys that the per-token kernel would fetch for every row by itself are staged in LDS
-// once for all of them (without a window every row's chunks start at key 0, so the rows share them).
+// once for all of them (without a window every row's blocks of 64 keys start at key 0, so the rows share
+// them; with chunks both kernels walk the blocks of 64 keys counted from key 0, from the one that holds
+// a row's first visible key, and mask what lies before it).
 #include "common.h"
 
 #define ATT_MAX_D 512
@@ -31,7 +34,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
                                const int32_t* __restrict__ block_tables, int table_stride,
                                const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
                                int num_q_heads, int num_kv_heads, int head_dim, int v_dim, int page_size, float scale,
-                               int window, const float* __restrict__ sinks, int32_t* error_flag) {
+                               int window, int chunk, const float* __restrict__ sinks, int32_t* error_flag) {
     __shared__ float q_s[ATT_MAX_D];
     __shared__ float p_s[NVA_WAVE];
     __shared__ int64_t v_off_s[NVA_WAVE];
@@ -42,7 +45,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
     const int kvh = h / (num_q_heads / num_kv_heads);
     const int seq = token_seq[t];
     const int pos = positions[t];
-    const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+    const int first = nva_first_key(pos, window, chunk);
     const int32_t* table = block_tables + (int64_t)seq * table_stride;
 
     const T* qrow = q + t * q_stride + (int64_t)h * head_dim;
@@ -56,11 +59,11 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
     const bool vec = head_dim % 8 == 0;
     const int vt = nva_v_tile(page_size);
 
-    for (int base = first; base <= pos; base += NVA_WAVE) {
+    for (int base = chunk > 0 ? first / NVA_WAVE * NVA_WAVE : first; base <= pos; base += NVA_WAVE) {
         const int j = base + lane;
         float s = -INFINITY;
         int64_t v_off = 0;
-        if (j <= pos) {
+        if (j <= pos && j >= first) {
             const int page = table[j / page_size];
             const int off = j % page_size;
             if (page < 0) {
@@ -159,7 +162,7 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
                              const int32_t* __restrict__ block_tables, int table_stride,
                              const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ kv_lens,
                              const int32_t* __restrict__ tiles, int num_q_heads, int num_kv_heads, int head_dim,
-                             int v_dim, int page_size, float scale, const float* __restrict__ sinks,
+                             int v_dim, int page_size, float scale, int chunk, const float* __restrict__ sinks,
                              int32_t* error_flag) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     __shared__ int64_t k_off_s[NVA_WAVE], v_off_s[NVA_WAVE];       // of a chunk's keys; -1: the key has no page
@@ -197,12 +200,14 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
         m_run[r] = sinks ? sinks[h] : -INFINITY, l_run[r] = sinks ? 1.f : 0.f;
     }
 
-    for (int base = 0; base <= last_pos; base += NVA_WAVE) {
+    // the first key any row of the tile reads (its first row's: the first key never decreases with the position)
+    const int first_any = nva_first_key(start + q0, 0, chunk);
+    for (int base = first_any / NVA_WAVE * NVA_WAVE; base <= last_pos; base += NVA_WAVE) {
         __syncthreads();                                             // the chunk before is done with (and q_s is written)
         if (tid < NVA_WAVE) {
             const int j = base + tid;
             int64_t k_off = -1, v_off = -1;
-            if (j <= last_pos) {
+            if (j <= last_pos && j >= first_any) {
                 const int page = table[j / page_size];
                 const int off = j % page_size;
                 if (page < 0) {
@@ -275,11 +280,12 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
         // its maximum, sum and accumulators as they are, bit for bit.
 #pragma unroll
         for (int quad = 0; quad < ROWS_PER_WAVE / 4; ++quad) {
-            int pos4[4], last4 = -1;
+            int pos4[4], first4[4], last4 = -1;
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 const int r = wave + ATT_TILED_WAVES * (4 * quad + t);
                 pos4[t] = r < rows ? start + q0 + r : -1;
+                first4[t] = r < rows ? nva_first_key(pos4[t], 0, chunk) : 0;
                 last4 = max(last4, pos4[t]);
             }
             if (base > last4) continue;                              // (the same for the whole wave)
@@ -316,7 +322,7 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 const int rr = 4 * quad + t;
-                const float s = base + lane <= pos4[t] && key_ok ? dot[t] * scale : -INFINITY;
+                const float s = base + lane <= pos4[t] && base + lane >= first4[t] && key_ok ? dot[t] * scale : -INFINITY;
                 const float m_new = fmaxf(m_run[rr], wave_max(s));
                 p[t] = (s == -INFINITY) ? 0.f : nva_exp(s - m_new);
                 const float correction = (m_run[rr] == -INFINITY) ? 0.f : nva_exp(m_run[rr] - m_new);
@@ -372,13 +378,14 @@ paged_attention_tiled_kernel(const T* __restrict__ q, int64_t q_stride, T* __res
 
 // The same attention for portions of prompts, 32 rows of a request to a workgroup: tiles is int32
 // [num_tiles][2] = (request, row tile of 32 queries), requests described by cu_seqlens_q and kv_lens as
-// for the matrix-core kernel.  No window, head sizes up to 128; returns 1 for what it does not take.
+// for the matrix-core kernel.  No window (chunks: yes), head sizes up to 128; returns 1 for what it does not take.
 NVA_EXPORT int NVA_NAME(nva_paged_attention_tiled)(
     const void* q, int64_t q_stride, void* out, int64_t out_stride, const void* k_cache, const void* v_cache,
     const int32_t* block_tables, int table_stride, const int32_t* cu_seqlens_q, const int32_t* kv_lens,
     const int32_t* tiles, int64_t num_tiles, int num_q_heads, int num_kv_heads, int head_dim, int v_dim,
-    int page_size, float scale, const float* sinks, int32_t* error_flag, hipStream_t stream) {
+    int page_size, float scale, int chunk, const float* sinks, int32_t* error_flag, hipStream_t stream) {
     if (num_tiles == 0) return 0;
+    if (chunk < 0) return nva_fail("paged_attention_tiled: negative chunk");
     if (head_dim <= 0 || head_dim > ATT_TILED_MAX_D || v_dim <= 0 || v_dim > ATT_TILED_MAX_D) {
         nva_fail("paged_attention_tiled: head sizes %d / %d are outside 1..%d", head_dim, v_dim, ATT_TILED_MAX_D);
         return 1;
@@ -399,7 +406,7 @@ NVA_EXPORT int NVA_NAME(nva_paged_attention_tiled)(
     hipLaunchKernelGGL(kernel, grid, dim3(ATT_TILED_WAVES * NVA_WAVE), lds, stream, (const elem_t*)q, q_stride,
                        (elem_t*)out, out_stride, (const elem_t*)k_cache, (const elem_t*)v_cache, block_tables,
                        table_stride, cu_seqlens_q, kv_lens, tiles, num_q_heads, num_kv_heads, head_dim, v_dim,
-                       page_size, scale, sinks, error_flag);
+                       page_size, scale, chunk, sinks, error_flag);
     return nva_check_launch("paged_attention_tiled");
 }
 
@@ -407,7 +414,7 @@ NVA_EXPORT int NVA_NAME(nva_paged_attention_generic)(
     const void* q, int64_t q_stride, void* out, int64_t out_stride, const void* k_cache, const void* v_cache,
     const int32_t* block_tables, int table_stride, const int32_t* token_seq, const int32_t* positions,
     int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, int v_dim, int page_size, float scale,
-    int window, const float* sinks, int32_t* error_flag, hipStream_t stream) {
+    int window, int chunk, const float* sinks, int32_t* error_flag, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || tokens > 0x7fffffff) return nva_fail("paged_attention: bad token count %lld", (long long)tokens);
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads || num_q_heads > 65535)
@@ -415,12 +422,12 @@ NVA_EXPORT int NVA_NAME(nva_paged_attention_generic)(
     if (head_dim <= 0 || head_dim > ATT_MAX_D || v_dim <= 0 || v_dim > ATT_MAX_D)
         return nva_fail("paged_attention: head sizes %d / %d are outside 1..%d", head_dim, v_dim, ATT_MAX_D);
     if (page_size <= 0 || table_stride <= 0) return nva_fail("paged_attention: bad page size or table width");
-    if (window < 0) return nva_fail("paged_attention: negative window");
+    if (window < 0 || chunk < 0) return nva_fail("paged_attention: negative window or chunk");
     dim3 grid((unsigned)tokens, (unsigned)num_q_heads);
     hipLaunchKernelGGL(paged_attention_generic_kernel<elem_t>, grid, dim3(NVA_WAVE), 0, stream, (const elem_t*)q,
                        q_stride, (elem_t*)out, out_stride, (const elem_t*)k_cache, (const elem_t*)v_cache,
                        block_tables, table_stride, token_seq, positions, num_q_heads, num_kv_heads, head_dim,
-                       v_dim, page_size, scale, window, sinks, error_flag);
+                       v_dim, page_size, scale, window, chunk, sinks, error_flag);
     return nva_check_launch("paged_attention_generic");
 }
 

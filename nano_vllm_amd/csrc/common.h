@@ -133,9 +133,10 @@ __device__ __forceinline__ float nva_exp(float x) {
 }
 
 // ---------------------------------------------------------------------------- gating
-// The activation of a gated feed-forward, by its code: 0 silu, 1 relu, 2 gelu (tanh form).
+// The activation of a feed-forward, by its code: 0 silu, 1 relu, 2 gelu (tanh form), 3 the square of relu.
 __device__ __forceinline__ float nva_gate_act(int act, float g) {
     if (act == 1) return fmaxf(g, 0.f);
+    if (act == 3) { const float r = fmaxf(g, 0.f); return r * r; }
     if (act == 2) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
     return g / (1.f + __expf(-g));
 }
@@ -213,6 +214,19 @@ __device__ __forceinline__ float nva_sum_over_rows(float x) {
     nva_lane_rows(x, a, b);
     nva_lane_halves(a + b, a, b);
     return a + b;
+}
+
+// ---------------------------------------------------------------------------- masks
+// The first key that a query at position pos reads: pos - window + 1 with a window (window > 0), the
+// start of its own chunk of `chunk` positions with chunks (chunk > 0; chunks are counted from the
+// request's position 0), the later of the two with both, else 0.  Never decreases with pos.
+__host__ __device__ __forceinline__ int nva_first_key(int pos, int window, int chunk) {
+    int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+    if (chunk > 0) {
+        const int c = pos / chunk * chunk;
+        first = c > first ? c : first;
+    }
+    return first;
 }
 
 // ---------------------------------------------------------------------------- cache layout

@@ -43,4 +43,21 @@ NVA_EXPORT int NVA_NAME(nva_gather_rows)(const void* table, int64_t table_stride
     return nva_check_launch("gather_rows");
 }
 
+// x <- x * factor over a float tensor of rows `stride` apart (logits times a model's constant).
+__global__ void scale_rows_kernel(float* __restrict__ x, int64_t stride, int64_t rows, int width, float factor) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * width) return;
+    float* p = x + (idx / width) * stride + idx % width;
+    *p = *p * factor;
+}
+
+NVA_EXPORT int NVA_NAME(nva_scale_rows)(float* x, int64_t stride, int64_t rows, int width, float factor, hipStream_t stream) {
+    if (rows == 0) return 0;
+    if (rows < 0 || width <= 0 || stride < width || !x) return nva_fail("scale_rows: bad arguments");
+    const int64_t total = rows * width;
+    hipLaunchKernelGGL(scale_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, x, stride, rows, width,
+                       factor);
+    return nva_check_launch("scale_rows");
+}
+
 NVA_DEFINE_LAST_ERROR(nva_embed)

@@ -1,0 +1,233 @@
+// A routed feed-forward (mixture of experts): the choice of experts, and the experts' products over
+// the tokens sorted by expert.  Nothing here asks the host how the tokens were shared out: every
+// kernel's launch depends on the number of tokens alone.
+//
+//   route     s = sigmoid(z) of the router's float logits z [tokens, E]; the experts form `group_count` equal
+//             groups of neighbours; a group's score is the sum of its two largest scores (of its one score
+//             where a group holds one expert); the `group_keep` groups with the largest scores stay; of
+//             their experts the `top` with the largest scores are chosen (equal scores: the lower number);
+//             ids [tokens, top], weights [tokens, top] = scale * s.
+//   plan      the pairs (token, choice) counted and sorted by expert: place[pair] = the pair's row among the
+//             sorted ones, rows[place] = pair; the sorted rows cut into tiles of MOE_BM rows of one expert:
+//             tile_expert[i], tile_row0[i], tile_rows[i], and their number.
+//   up        h[row] = act(x[token of row] Wu_e^T)         rows sorted by expert, a tile of rows and 64 outputs
+//   down      o[row] = h[row] Wd_e^T                       to a workgroup
+//   combine   y[token] = sum over its choices of weight * o[place] (+ add[token])
+//
+// The products are float sums over k in ascending order, one chain per output, so a token's result does
+// not depend on what else is in the batch or on where its row fell among the sorted ones; operands and
+// results are elements (rounded once), the combination is float.
+#include "common.h"
+
+#define MOE_BM 32
+#define MOE_BN 64
+#define MOE_BK 32
+#define MOE_MAX_EXPERTS 1024
+
+__global__ void __launch_bounds__(NVA_WAVE)
+moe_route_kernel(const float* __restrict__ logits, int64_t stride, int experts, int top, int group_count, int group_keep,
+                 float scale, int32_t* __restrict__ ids, float* __restrict__ weights) {
+    __shared__ float s_s[MOE_MAX_EXPERTS];
+    __shared__ float g_s[MOE_MAX_EXPERTS];           // group scores; -inf once taken
+    __shared__ unsigned char open_s[MOE_MAX_EXPERTS];
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x;
+    for (int e = lane; e < experts; e += NVA_WAVE) s_s[e] = 1.f / (1.f + expf(-logits[t * stride + e]));
+    __syncthreads();
+    const int per = experts / group_count;
+    for (int g = lane; g < group_count; g += NVA_WAVE) {
+        float a = -INFINITY, b = -INFINITY;          // the two largest of the group
+        for (int i = 0; i < per; ++i) {
+            const float v = s_s[g * per + i];
+            if (v > a) { b = a; a = v; } else if (v > b) b = v;
+        }
+        g_s[g] = per > 1 ? a + b : a;
+    }
+    for (int e = lane; e < experts; e += NVA_WAVE) open_s[e] = 0;
+    __syncthreads();
+    if (lane == 0) {
+        for (int k = 0; k < group_keep; ++k) {
+            int best = 0;
+            for (int g = 1; g < group_count; ++g)
+                if (g_s[g] > g_s[best]) best = g;
+            g_s[best] = -INFINITY;
+            for (int i = 0; i < per; ++i) open_s[best * per + i] = 1;
+        }
+        for (int k = 0; k < top; ++k) {
+            int best = -1;
+            for (int e = 0; e < experts; ++e)
+                if (open_s[e] && (best < 0 || s_s[e] > s_s[best])) best = e;
+            open_s[best] = 0;
+            ids[t * top + k] = best;
+            weights[t * top + k] = scale * s_s[best];
+        }
+    }
+}
+
+// One workgroup.  Counts and offsets live in LDS; pairs is tokens * top.  Where a pair falls among the rows
+// of its expert depends on the order in which the threads arrive; no result does, since every row of the
+// products is computed by itself.
+__global__ void __launch_bounds__(1024)
+moe_plan_kernel(const int32_t* __restrict__ ids, int64_t pairs, int experts, int32_t* __restrict__ place,
+                int32_t* __restrict__ rows, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
+                int32_t* __restrict__ tile_rows, int32_t* __restrict__ num_tiles) {
+    __shared__ int count_s[MOE_MAX_EXPERTS], cursor_s[MOE_MAX_EXPERTS], begin_s[MOE_MAX_EXPERTS], tile0_s[MOE_MAX_EXPERTS];
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) count_s[e] = cursor_s[e] = 0;
+    __syncthreads();
+    for (int64_t i = threadIdx.x; i < pairs; i += blockDim.x) atomicAdd(&count_s[ids[i]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0, tiles = 0;
+        for (int e = 0; e < experts; ++e) {
+            begin_s[e] = at;
+            tile0_s[e] = tiles;
+            at += count_s[e];
+            tiles += (count_s[e] + MOE_BM - 1) / MOE_BM;
+        }
+        num_tiles[0] = tiles;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) {
+        const int n = count_s[e];
+        for (int i = 0; i * MOE_BM < n; ++i) {
+            tile_expert[tile0_s[e] + i] = e;
+            tile_row0[tile0_s[e] + i] = begin_s[e] + i * MOE_BM;
+            tile_rows[tile0_s[e] + i] = min(MOE_BM, n - i * MOE_BM);
+        }
+    }
+    for (int64_t i = threadIdx.x; i < pairs; i += blockDim.x) {
+        const int e = ids[i];
+        const int r = begin_s[e] + atomicAdd(&cursor_s[e], 1);
+        place[i] = r;
+        rows[r] = (int32_t)i;
+    }
+}
+
+// Tile product: out[row0 + r, n0 + c] = f(sum_k a[src(row0 + r), k] * w[e * n + n0 + c, k]).
+// UP: src = token of the pair (rows[row] / top), f = act; else src = the row itself, f = identity.
+template <typename T, bool UP>
+__global__ void __launch_bounds__(256)
+moe_tile_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w, int n, int k,
+                const int32_t* __restrict__ rows, int top, const int32_t* __restrict__ tile_expert,
+                const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ tile_rows,
+                const int32_t* __restrict__ num_tiles, int act, T* __restrict__ out, int64_t out_stride) {
+    __shared__ float a_s[MOE_BM][MOE_BK + 1];
+    __shared__ float w_s[MOE_BN][MOE_BK + 1];
+    __shared__ int src_s[MOE_BM];
+    const int tile = blockIdx.x;
+    if (tile >= num_tiles[0]) return;
+    const int e = tile_expert[tile], row0 = tile_row0[tile], nrows = tile_rows[tile];
+    const int n0 = blockIdx.y * MOE_BN;
+    const int tid = threadIdx.x;
+    if (tid < MOE_BM) src_s[tid] = tid < nrows ? (UP ? rows[row0 + tid] / top : row0 + tid) : -1;
+    __syncthreads();
+    const T* we = w + (int64_t)e * n * k;
+    const int ty = tid / 16, tx = tid % 16;          // rows ty, ty + 16; columns tx + 16 j
+    float acc[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    for (int k0 = 0; k0 < k; k0 += MOE_BK) {
+        for (int i = tid; i < MOE_BM * MOE_BK; i += 256) {
+            const int r = i / MOE_BK, c = i % MOE_BK;
+            a_s[r][c] = src_s[r] >= 0 && k0 + c < k ? to_float(a[(int64_t)src_s[r] * a_stride + k0 + c]) : 0.f;
+        }
+        for (int i = tid; i < MOE_BN * MOE_BK; i += 256) {
+            const int r = i / MOE_BK, c = i % MOE_BK;
+            w_s[r][c] = n0 + r < n && k0 + c < k ? to_float(we[(int64_t)(n0 + r) * k + k0 + c]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < MOE_BK; ++c) {
+            const float a0 = a_s[ty][c], a1 = a_s[ty + 16][c];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float b = w_s[tx + 16 * j][c];
+                acc[0][j] += a0 * b;
+                acc[1][j] += a1 * b;
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int r = ty + 16 * i;
+        if (r >= nrows) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = n0 + tx + 16 * j;
+            if (c < n) out[(int64_t)(row0 + r) * out_stride + c] = from_float<T>(UP ? nva_gate_act(act, acc[i][j]) : acc[i][j]);
+        }
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_combine_kernel(const T* __restrict__ o, int64_t o_stride, const int32_t* __restrict__ place,
+                   const float* __restrict__ weights, int top, const T* __restrict__ add, int64_t add_stride,
+                   T* __restrict__ y, int64_t y_stride, int width) {
+    const int64_t t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= width) return;
+    float sum = 0.f;
+    for (int c = 0; c < top; ++c) sum += weights[t * top + c] * to_float(o[(int64_t)place[t * top + c] * o_stride + i]);
+    if (add) sum += to_float(add[t * add_stride + i]);
+    y[t * y_stride + i] = from_float<T>(sum);
+}
+
+NVA_EXPORT int NVA_NAME(nva_moe_route)(const float* logits, int64_t stride, int64_t tokens, int experts, int top,
+                                       int group_count, int group_keep, float scale, int32_t* ids, float* weights,
+                                       hipStream_t stream) {
+    if (tokens == 0) return 0;
+    if (tokens < 0 || tokens > 0x7fffffff || experts <= 0 || experts > MOE_MAX_EXPERTS)
+        return nva_fail("moe_route: bad counts tokens=%lld experts=%d (up to %d)", (long long)tokens, experts, MOE_MAX_EXPERTS);
+    if (group_count <= 0 || experts % group_count || group_keep <= 0 || group_keep > group_count || top <= 0 ||
+        top > group_keep * (experts / group_count))
+        return nva_fail("moe_route: %d of %d experts in %d groups of which %d stay", top, experts, group_count, group_keep);
+    if (!logits || !ids || !weights || stride < experts) return nva_fail("moe_route: a tensor is missing");
+    hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)tokens), dim3(NVA_WAVE), 0, stream, logits, stride, experts, top,
+                       group_count, group_keep, scale, ids, weights);
+    return nva_check_launch("moe_route");
+}
+
+// Rows of a tile of the experts' products (the plan's arrays are sized with it).
+NVA_EXPORT int NVA_NAME(nva_moe_tile_rows)() { return MOE_BM; }
+
+// x [tokens, k] elements; ids, weights [tokens, top]; up [E * ff, k], down [E * k, ff] elements; add [tokens, k] or null.
+// Scratch: place, rows int32 [tokens * top]; tiles int32 [3 * max_tiles + 1] with max_tiles = tokens * top / MOE_BM + E
+// (expert, first row, rows of every tile, then their number); hidden [tokens * top, ff], outs [tokens * top, k] elements.
+NVA_EXPORT int NVA_NAME(nva_moe_experts)(const void* x, int64_t x_stride, const int32_t* ids, const float* weights,
+                                         int64_t tokens, int top, int experts, int k, int ff, const void* up,
+                                         const void* down, int act, const void* add, int64_t add_stride, int32_t* place,
+                                         int32_t* rows, int32_t* tiles, int64_t max_tiles, void* hidden, void* outs, void* y,
+                                         int64_t y_stride, hipStream_t stream) {
+    if (tokens == 0) return 0;
+    const int64_t pairs = tokens * top;
+    if (tokens < 0 || top <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || k <= 0 || ff <= 0 || pairs > 0x7fffffff)
+        return nva_fail("moe_experts: bad sizes tokens=%lld top=%d experts=%d k=%d ff=%d", (long long)tokens, top, experts, k, ff);
+    if (max_tiles < pairs / MOE_BM + experts || max_tiles > 0x7fffffff)
+        return nva_fail("moe_experts: room for %lld tiles, %lld may be needed", (long long)max_tiles, (long long)(pairs / MOE_BM + experts));
+    if (act < 0 || act > 3) return nva_fail("moe_experts: unknown activation %d", act);
+    if (!x || !ids || !weights || !up || !down || !place || !rows || !tiles || !hidden || !outs || !y)
+        return nva_fail("moe_experts: a tensor is missing");
+    int32_t* tile_expert = tiles;
+    int32_t* tile_row0 = tiles + max_tiles;
+    int32_t* tile_rows = tiles + 2 * max_tiles;
+    int32_t* num_tiles = tiles + 3 * max_tiles;
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, place, rows, tile_expert,
+                       tile_row0, tile_rows, num_tiles);
+    if ((ff + MOE_BN - 1) / MOE_BN > 65535 || (k + MOE_BN - 1) / MOE_BN > 65535) return nva_fail("moe_experts: too wide");
+    hipLaunchKernelGGL((moe_tile_kernel<elem_t, true>), dim3((unsigned)max_tiles, (ff + MOE_BN - 1) / MOE_BN), dim3(256), 0,
+                       stream, (const elem_t*)x, x_stride, (const elem_t*)up, ff, k, rows, top, tile_expert, tile_row0,
+                       tile_rows, num_tiles, act, (elem_t*)hidden, (int64_t)ff);
+    hipLaunchKernelGGL((moe_tile_kernel<elem_t, false>), dim3((unsigned)max_tiles, (k + MOE_BN - 1) / MOE_BN), dim3(256), 0,
+                       stream, (const elem_t*)hidden, (int64_t)ff, (const elem_t*)down, k, ff, rows, top, tile_expert,
+                       tile_row0, tile_rows, num_tiles, act, (elem_t*)outs, (int64_t)k);
+    for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
+        const unsigned nt = (unsigned)((tokens - t0) < 65535 ? (tokens - t0) : 65535);
+        hipLaunchKernelGGL((moe_combine_kernel<elem_t>), dim3((k + 255) / 256, nt), dim3(256), 0, stream, (const elem_t*)outs,
+                           (int64_t)k, place + t0 * top, weights + t0 * top, top,
+                           add ? (const elem_t*)add + t0 * add_stride : nullptr, add_stride, (elem_t*)y + t0 * y_stride,
+                           y_stride, k);
+    }
+    return nva_check_launch("moe_experts");
+}
+
+NVA_DEFINE_LAST_ERROR(nva_moe)

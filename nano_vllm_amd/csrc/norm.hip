@@ -248,4 +248,95 @@ NVA_EXPORT int NVA_NAME(nva_stream_rms_norm)(const void* a, int64_t a_stride, co
     return nva_check_launch("stream_rms_norm");
 }
 
+// ---------------------------------------------------------------------------- Dynamic Tanh on the float stream
+//     r <- r + a + b   (first: r <- a + b)        a, b elements or absent
+//     y = tanh(alpha * r) * w + c                  alpha one float read on the device, w and c float vectors
+// No mean and no variance: every entry by itself.  All float, rounded once.
+template <typename T>
+__global__ void __launch_bounds__(256)
+stream_dyt_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ b, int64_t b_stride, float* residual,
+                  int64_t r_stride, int first, const float* __restrict__ weight, const float* __restrict__ bias,
+                  const float* __restrict__ alpha, T* __restrict__ y, int64_t y_stride, int width) {
+    const int64_t row = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= width) return;
+    float* rr = residual + row * r_stride;
+    float s = first ? 0.f : rr[i];
+    float add = 0.f;
+    if (a) add = to_float(a[row * a_stride + i]);
+    if (b) add += to_float(b[row * b_stride + i]);
+    s += add;
+    if (a || b || first) rr[i] = s;
+    y[row * y_stride + i] = from_float<T>(tanhf(alpha[0] * s) * weight[i] + bias[i]);
+}
+
+NVA_EXPORT int NVA_NAME(nva_stream_dyt)(const void* a, int64_t a_stride, const void* b, int64_t b_stride, float* residual,
+                                        int64_t r_stride, int first, const float* weight, const float* bias,
+                                        const float* alpha, void* y, int64_t y_stride, int64_t rows, int width,
+                                        hipStream_t stream) {
+    if (rows == 0) return 0;
+    if (rows < 0 || width <= 0) return nva_fail("stream_dyt: bad shape rows=%lld width=%d", (long long)rows, width);
+    if (!residual || !y || !weight || !bias || !alpha) return nva_fail("stream_dyt: residual, output, weight, bias and alpha are needed");
+    if (first && !a) return nva_fail("stream_dyt: the stream starts with an addend");
+    for (int64_t r0 = 0; r0 < rows; r0 += 65535) {
+        const unsigned nr = (unsigned)((rows - r0) < 65535 ? (rows - r0) : 65535);
+        hipLaunchKernelGGL((stream_dyt_kernel<elem_t>), dim3((width + 255) / 256, nr), dim3(256), 0, stream,
+                           a ? (const elem_t*)a + r0 * a_stride : nullptr, a_stride,
+                           b ? (const elem_t*)b + r0 * b_stride : nullptr, b_stride, residual + r0 * r_stride, r_stride, first,
+                           weight, bias, alpha, (elem_t*)y + r0 * y_stride, y_stride, width);
+    }
+    return nva_check_launch("stream_dyt");
+}
+
+// ---------------------------------------------------------------------------- two normed inputs, averaged
+//     y = ( a * rsqrt(mean(a^2) + eps) * wa  +  b * rsqrt(mean(b^2) + eps) * wb ) / 2
+// a, b elements [rows, width] (each may come as the partial sums of a split product), wa, wb float [width].
+template <typename T>
+__global__ void __launch_bounds__(1024)
+pair_norm_mean_kernel(const T* __restrict__ a, int64_t a_stride, PartialInput pa, const float* __restrict__ wa,
+                      const T* __restrict__ b, int64_t b_stride, PartialInput pb, const float* __restrict__ wb,
+                      T* __restrict__ y, int64_t y_stride, int width, float eps) {
+    extern __shared__ __attribute__((aligned(16))) float row_s[];       // a's row, then b's
+    __shared__ float scratch[16];
+    const int64_t row = blockIdx.x;
+    float sa = 0.f, sb = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float x = pa.sums ? partial_value<T>(pa, row, width, i) : to_float(a[row * a_stride + i]);
+        const float z = pb.sums ? partial_value<T>(pb, row, width, i) : to_float(b[row * b_stride + i]);
+        row_s[i] = x;
+        row_s[width + i] = z;
+        sa += x * x;
+        sb += z * z;
+    }
+    sa = block_sum(sa, scratch);
+    sb = block_sum(sb, scratch);
+    const float ra = rsqrtf(sa / (float)width + eps), rb = rsqrtf(sb / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += blockDim.x)
+        y[row * y_stride + i] = from_float<T>(0.5f * (row_s[i] * ra * wa[i] + row_s[width + i] * rb * wb[i]));
+}
+
+NVA_EXPORT int NVA_NAME(nva_pair_norm_mean)(const void* a, int64_t a_stride, const float* a_sums, int a_splits,
+                                            int64_t a_split_stride, const void* a_bias, const float* wa, const void* b,
+                                            int64_t b_stride, const float* b_sums, int b_splits, int64_t b_split_stride,
+                                            const void* b_bias, const float* wb, void* y, int64_t y_stride, int64_t rows,
+                                            int width, float eps, hipStream_t stream) {
+    if (rows == 0) return 0;
+    if (rows < 0 || rows > 0x7fffffff || width <= 0 || width > 16 * 1024)
+        return nva_fail("pair_norm_mean: bad shape rows=%lld width=%d", (long long)rows, width);
+    if ((!a && !a_sums) || (!b && !b_sums) || !wa || !wb || !y) return nva_fail("pair_norm_mean: both inputs, both weights and the output are needed");
+    const PartialInput pa{a_sums, a_splits, a_split_stride, a_bias}, pb{b_sums, b_splits, b_split_stride, b_bias};
+    const int threads = width >= 2048 ? 512 : width >= 512 ? 256 : 128;
+    auto kernel = pair_norm_mean_kernel<elem_t>;
+    const size_t lds = 2 * (size_t)width * sizeof(float);
+    static bool raised = false;
+    if (!raised && lds > 48 * 1024) {
+        if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024) != hipSuccess)
+            return nva_fail("pair_norm_mean: cannot have %zu bytes of LDS", lds);
+        raised = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)rows), dim3(threads), lds, stream, (const elem_t*)a, a_stride, pa, wa,
+                       (const elem_t*)b, b_stride, pb, wb, (elem_t*)y, y_stride, width, eps);
+    return nva_check_launch("pair_norm_mean");
+}
+
 NVA_DEFINE_LAST_ERROR(nva_norm)

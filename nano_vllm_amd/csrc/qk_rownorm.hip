@@ -5,6 +5,8 @@
 //     q <- q / sqrt(mean(q^2) + eps) * wq * temp(p)        mean over all Hq * D entries of the token's q
 //     k <- k / sqrt(mean(k^2) + eps) * wk                  mean over all Hkv * D entries
 //     temp(p) = 1 + coef * ln(floor((p + 1) / every) + 1)  (coef 0: no temperature)
+//     q, k <- rotation of the first R channels of every head, pairs (i, i + R/2), by the token's row of
+//             rot_table (R/2 cosines, then R/2 sines; null: no rotation), after norm and temperature
 //     cache <- k, v                                        at the token's slot (slot < 0: nothing is written)
 //
 // The row is the packed projection [q | k | v] of Hq * D, Hkv * D and Hkv * DV entries, biases added
@@ -22,6 +24,7 @@ qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput 
                         int64_t q_stride, int num_heads, int num_kv_heads, int head_dim, int v_dim,
                         const void* __restrict__ q_weight, const void* __restrict__ k_weight, int w_is_f32, float eps,
                         const int32_t* __restrict__ positions, float temp_coef, int temp_every,
+                        const float* __restrict__ rot_table, int rot,
                         const int32_t* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
                         int page_size) {
     extern __shared__ __attribute__((aligned(16))) float row_s[];      // the token's row, as float
@@ -46,21 +49,31 @@ qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput 
     float q_scale = q_weight ? rsqrtf(sq / (float)qd + eps) : 1.f;
     if (temp_coef != 0.f) q_scale *= 1.f + temp_coef * logf((float)steps + 1.f);
     T* qrow = q_out + t * q_stride;
-    for (int i = tid; i < qd; i += blockDim.x) {
-        const float w = !q_weight ? 1.f : w_is_f32 ? static_cast<const float*>(q_weight)[i]
-                                                   : to_float(static_cast<const T*>(q_weight)[i]);
-        qrow[i] = from_float<T>(row_s[i] * q_scale * w);
-    }
+    const float* rot_row = rot_table ? rot_table + t * (int64_t)rot : nullptr;
+    const int half = rot / 2;
+    auto weight_of = [&](const void* w, int i) -> float {
+        return !w ? 1.f : w_is_f32 ? static_cast<const float*>(w)[i] : to_float(static_cast<const T*>(w)[i]);
+    };
+    // entry i of a projection that starts at `at` in the row, scaled and weighted, then turned with its partner
+    auto prepared = [&](int at, int i, float scale, const void* w) -> float {
+        const float x = row_s[at + i] * scale * weight_of(w, i);
+        const int d = i % head_dim;
+        if (!rot_row || d >= rot) return x;
+        const int f = d < half ? d : d - half;
+        const int j = d < half ? i + half : i - half;
+        const float y = row_s[at + j] * scale * weight_of(w, j);
+        const float c = rot_row[f], sn = rot_row[half + f];
+        return d < half ? x * c - y * sn : x * c + y * sn;
+    };
+    for (int i = tid; i < qd; i += blockDim.x) qrow[i] = from_float<T>(prepared(0, i, q_scale, q_weight));
     if (!kd || slot < 0 || !k_cache) return;
     const float k_scale = k_weight ? rsqrtf(sk / (float)kd + eps) : 1.f;
     const int page = slot / page_size, off = slot % page_size;
     const int vt = nva_v_tile(page_size);
     for (int i = tid; i < kd; i += blockDim.x) {
-        const float w = !k_weight ? 1.f : w_is_f32 ? static_cast<const float*>(k_weight)[i]
-                                                   : to_float(static_cast<const T*>(k_weight)[i]);
         const int g = i / head_dim, d = i % head_dim;
         k_cache[(((int64_t)page * num_kv_heads + g) * page_size + off) * head_dim + d] =
-            from_float<T>(row_s[qd + i] * k_scale * w);
+            from_float<T>(prepared(qd, i, k_scale, k_weight));
     }
     for (int i = tid; i < vd; i += blockDim.x) {
         const int g = i / v_dim, d = i % v_dim;
@@ -73,14 +86,15 @@ qk_rownorm_store_kernel(const T* __restrict__ qkv, int64_t stride, PartialInput 
 // partial sums [splits][tokens][width] of the projection with its bias, which are added up here.
 // q_out: [tokens, Hq * D] with rows q_stride apart (it may be qkv itself: q is then rewritten in place).
 // q_weight [Hq * D], k_weight [Hkv * D]: both or none.  positions are needed with a temperature.
+// rot_table: float [tokens, rot], a row per token of this call, or null.
 // slots (with the caches) may be null: nothing is stored then.  num_kv_heads 0: the row holds q only.
 NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(const void* qkv, int64_t stride, const float* sums, int splits,
                                               int64_t split_stride, const void* bias, void* q_out, int64_t q_stride,
                                               int64_t tokens, int num_heads, int num_kv_heads,
                                               int head_dim, int v_dim, const void* q_weight, const void* k_weight,
                                               int w_is_f32, float eps, const int32_t* positions, float temp_coef,
-                                              int temp_every, const int32_t* slots, void* k_cache, void* v_cache,
-                                              int page_size, hipStream_t stream) {
+                                              int temp_every, const float* rot_table, int rot, const int32_t* slots,
+                                              void* k_cache, void* v_cache, int page_size, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || tokens > 0x7fffffff) return nva_fail("qk_rownorm_store: bad token count %lld", (long long)tokens);
     if (num_heads <= 0 || num_kv_heads < 0 || head_dim <= 0 || v_dim <= 0)
@@ -96,6 +110,8 @@ NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(const void* qkv, int64_t stride, c
         return nva_fail("qk_rownorm_store: give both norm weights or none");
     if (temp_coef != 0.f && (!positions || temp_every <= 0))
         return nva_fail("qk_rownorm_store: a query temperature needs positions and a positive step");
+    if (rot_table && (rot <= 0 || rot % 2 || rot > head_dim))
+        return nva_fail("qk_rownorm_store: %d rotated channels of a head of %d", rot, head_dim);
     if ((k_cache || v_cache) && (!k_cache || !v_cache || !slots || page_size <= 0 || !num_kv_heads))
         return nva_fail("qk_rownorm_store: storing needs both caches, the slots and the page size");
     auto kernel = qk_rownorm_store_kernel<elem_t>;
@@ -111,7 +127,7 @@ NVA_EXPORT int NVA_NAME(nva_qk_rownorm_store)(const void* qkv, int64_t stride, c
     const int threads = tokens <= 64 && width >= 2048 ? 1024 : 256;
     hipLaunchKernelGGL(kernel, dim3((unsigned)tokens), dim3(threads), lds, stream, (const elem_t*)qkv, stride, part,
                        (elem_t*)q_out, q_stride, num_heads, num_kv_heads, head_dim, v_dim, q_weight, k_weight, w_is_f32, eps,
-                       positions, temp_coef, temp_every, slots, (elem_t*)k_cache, (elem_t*)v_cache, page_size);
+                       positions, temp_coef, temp_every, rot_table, rot_table ? rot : 0, slots, (elem_t*)k_cache, (elem_t*)v_cache, page_size);
     return nva_check_launch("qk_rownorm_store");
 }
 

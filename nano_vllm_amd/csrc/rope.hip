@@ -343,4 +343,31 @@ NVA_EXPORT int NVA_NAME(nva_qk_norm_rope_store_of_partials)(
                      slots, k_cache, v_cache, page_size, stream);
 }
 
+// ---------------------------------------------------------------------------- the step's own table
+// table[t] = cos(p_t * f_i) for i < half, then sin(p_t * f_i): the rotation of the step's tokens at their
+// positions p_t, read on the device.  The product is one float multiplication and the sine and cosine
+// are the accurate routines in both builds: the angles are part of the model.
+__global__ void rotary_step_table_kernel(const float* __restrict__ inv_freq, int half, const int32_t* __restrict__ positions,
+                                         int64_t tokens, float* __restrict__ table) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= tokens * half) return;
+    const int64_t t = idx / half;
+    const int i = (int)(idx % half);
+    const float angle = (float)positions[t] * inv_freq[i];
+    float sn, cs;
+    sincosf(angle, &sn, &cs);
+    table[t * 2 * half + i] = cs;
+    table[t * 2 * half + half + i] = sn;
+}
+
+NVA_EXPORT int NVA_NAME(nva_rotary_step_table)(const float* inv_freq, int half, const int32_t* positions, int64_t tokens,
+                                               float* table, hipStream_t stream) {
+    if (tokens == 0) return 0;
+    if (tokens < 0 || half <= 0 || !inv_freq || !positions || !table) return nva_fail("rotary_step_table: bad arguments");
+    const int64_t total = tokens * half;
+    hipLaunchKernelGGL(rotary_step_table_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, inv_freq, half,
+                       positions, tokens, table);
+    return nva_check_launch("rotary_step_table");
+}
+
 NVA_DEFINE_LAST_ERROR(nva_rope)

@@ -1,0 +1,337 @@
+// A selective state-space layer with a scalar decay per head and token, after its input projection.
+//
+// The projection's row is [z | x B C | dt]: z and x of H * P channels (H heads of P), B and C of G * N
+// (G groups, N state rows; head h reads group h / (H / G)), dt of H.  Per request the layer keeps, in
+// the request's slot, S [H, N, P] and the last K - 1 inputs of the convolution [C, K - 1] (C = H * P +
+// 2 G N channels), both float, taken as zero where the request starts (seq_starts == 0).
+//
+//   conv      u_t[c] = silu(b[c] + sum_j w[c][j] * in_(t - (K - 1) + j)[c])          over x, B and C; in before the
+//                                                                                    request's start is zero
+//   step      dt_t[h] = softplus(dt_raw + dt_bias[h]);  a_t[h] = exp(-exp(A_log[h]) * dt_t[h])
+//   state     S_t = a_t S_(t-1) + dt_t B_t x_t^T;  y_t = S_t^T C_t + D[h] x_t
+//   finish    y <- y * silu(z), then y / sqrt(mean(y^2) + eps) * w in norm_groups equal parts of the H * P channels
+//
+// The convolution's sums and silu are float and rounded once to the element type; everything after
+// (step sizes, decays, the state, the read-out, gate and norm) is float with the accurate exponential
+// and logarithm in both builds, rounded once at the output.
+//
+// Kernels: conv (a thread per token and channel; a request that brings one token also shifts its kept
+// inputs), conv_state (the kept inputs of requests that bring a portion), scan, finish.  The scan gives
+// every thread one column of S (all N rows, in registers), so the read-out needs no exchange between
+// threads; B and C of a token are staged in LDS for the wave.  A long portion is cut into blocks that
+// run side by side, each from a zero state (the first from the request's); a pass over the blocks makes
+// every block's true state at its end, E_b = exp(sum of the block's log-decays) E_(b-1) + U_b, and a
+// second pass adds what the state before a block contributes, exp(log-decay up to t) E_(b-1)^T C_t.
+#include "common.h"
+
+#define SSD_MAX_TAPS 16
+
+__device__ __forceinline__ float ssd_silu(float x) { return x / (1.f + expf(-x)); }
+__device__ __forceinline__ float ssd_softplus(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+
+// ---------------------------------------------------------------------------- convolution
+template <typename T>
+__global__ void __launch_bounds__(256)
+ssd_conv_kernel(const T* __restrict__ proj, int64_t stride, int col0, int channels, int taps,
+                const T* __restrict__ conv_w, const T* __restrict__ conv_b, float* __restrict__ conv_state,
+                const int32_t* __restrict__ token_seq, const int32_t* __restrict__ cu_seqlens,
+                const int32_t* __restrict__ seq_starts, const int32_t* __restrict__ state_slots,
+                T* __restrict__ out) {
+    const int64_t t = blockIdx.x;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= channels) return;
+    const int s = token_seq[t];
+    const int begin = cu_seqlens[s], n = cu_seqlens[s + 1] - begin;
+    const int i = (int)(t - begin);                      // the token's place in its request's portion
+    const bool carried = seq_starts[s] > 0;
+    const int hist = taps - 1;
+    float* kept = conv_state + ((int64_t)state_slots[s] * channels + c) * hist;
+    float in[SSD_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < SSD_MAX_TAPS; ++j) {
+        if (j >= taps) break;
+        const int src = i - (hist - j);                  // place in the portion of tap j's input
+        if (src >= 0) in[j] = to_float(proj[(t - (hist - j)) * stride + col0 + c]);
+        else in[j] = carried ? kept[i + j] : 0.f;        // hist + src = i + j
+    }
+    float sum = to_float(conv_b[c]);
+#pragma unroll
+    for (int j = 0; j < SSD_MAX_TAPS; ++j) {
+        if (j >= taps) break;
+        sum += to_float(conv_w[(int64_t)c * taps + j]) * in[j];
+    }
+    out[t * channels + c] = from_float<T>(ssd_silu(sum));
+    if (n == 1) {                                        // a single token: the kept inputs move on by one
+#pragma unroll
+        for (int j = 0; j < SSD_MAX_TAPS - 1; ++j) {
+            if (j >= hist) break;
+            kept[j] = in[j + 1];
+        }
+    }
+}
+
+// The kept inputs of the requests that bring more than one token: the last K - 1 inputs of the portion,
+// or, where the portion is shorter, the old ones moved on.  A thread per (request, channel) reads all it
+// needs before it writes.
+template <typename T>
+__global__ void __launch_bounds__(256)
+ssd_conv_state_kernel(const T* __restrict__ proj, int64_t stride, int col0, int channels, int taps,
+                      float* __restrict__ conv_state, const int32_t* __restrict__ cu_seqlens,
+                      const int32_t* __restrict__ seq_starts, const int32_t* __restrict__ state_slots, int first_seq) {
+    const int s = first_seq + blockIdx.y;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= channels) return;
+    const int begin = cu_seqlens[s], n = cu_seqlens[s + 1] - begin;
+    if (n <= 1) return;
+    const bool carried = seq_starts[s] > 0;
+    const int hist = taps - 1;
+    float* kept = conv_state + ((int64_t)state_slots[s] * channels + c) * hist;
+    float next[SSD_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < SSD_MAX_TAPS - 1; ++j) {
+        if (j >= hist) break;
+        const int src = n - hist + j;
+        if (src >= 0) next[j] = to_float(proj[(int64_t)(begin + src) * stride + col0 + c]);
+        else next[j] = carried ? kept[j + n] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < SSD_MAX_TAPS - 1; ++j) {
+        if (j >= hist) break;
+        kept[j] = next[j];
+    }
+}
+
+// ---------------------------------------------------------------------------- the recurrence
+// One wave per (unit, head, 64 columns of S).  A unit is a run of tokens of one request: a whole
+// request's tokens of this step (units == null: unit u is request first_seq + u), or a block of a
+// portion (units[u] = request, first token within the portion, tokens, blocks of the portion).
+// mode 0: from the request's state (zero at its start) to its new state, which is written back.
+// mode 1 (blocks): a portion's first block starts from the request's state, the others from zero; every
+//         block leaves its end state in block_states[u] and its tokens' log-decays, summed from the block's
+//         start, in cum[t, h]; the request's state is not written.
+// mode 2 (blocks, second pass): the blocks after a portion's first add exp(cum_t) E^T C_t to y, E the true
+//         state before the block (block_states[u - 1] after the pass over the blocks).
+template <typename T, int NMAX>
+__global__ void __launch_bounds__(NVA_WAVE)
+ssd_scan_kernel(const T* __restrict__ proj, int64_t stride, int dt_col, const T* __restrict__ conv, int channels,
+                int heads, int vdim, int n_state, int groups, const float* __restrict__ dt_bias,
+                const float* __restrict__ a_log, const float* __restrict__ d_skip, float* __restrict__ state,
+                const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_starts,
+                const int32_t* __restrict__ state_slots, int first_seq, const int32_t* __restrict__ units, int mode,
+                float* __restrict__ block_states, float* __restrict__ cum, float* __restrict__ y) {
+    __shared__ float b_s[NMAX], c_s[NMAX];
+    const int u = blockIdx.z, h = blockIdx.y;
+    const int p = blockIdx.x * NVA_WAVE + threadIdx.x;
+    const bool mine = p < vdim;
+    int s, t0, n, first_block = 1;
+    if (units) {
+        s = first_seq + units[4 * u];
+        t0 = cu_seqlens[s] + units[4 * u + 1];
+        n = units[4 * u + 2];
+        first_block = units[4 * u + 1] == 0;
+    } else {
+        s = first_seq + u;
+        t0 = cu_seqlens[s];
+        n = cu_seqlens[s + 1] - t0;
+    }
+    if (mode == 2 && first_block) return;
+    const int inner = heads * vdim, gn = groups * n_state;
+    const int g = h / (heads / groups);
+    const T* b_col = conv + inner + g * n_state;
+    const T* c_col = b_col + gn;
+    float* own = state + (((int64_t)state_slots[s] * heads + h) * n_state) * vdim + p;
+    float* block = block_states ? block_states + (((int64_t)u * heads + h) * n_state) * vdim + p : nullptr;
+
+    float S[NMAX];
+    if (mode == 2) {
+        const float* before = block - (int64_t)heads * n_state * vdim;       // the unit before: the block before
+#pragma unroll
+        for (int i = 0; i < NMAX; ++i) S[i] = mine && i < n_state ? before[(int64_t)i * vdim] : 0.f;
+    } else {
+        const bool carried = first_block && seq_starts[s] > 0;
+#pragma unroll
+        for (int i = 0; i < NMAX; ++i) S[i] = carried && mine && i < n_state ? own[(int64_t)i * vdim] : 0.f;
+    }
+    const float rate = -expf(a_log[h]), bias = dt_bias[h], skip = d_skip[h];
+    float log_decay = 0.f;
+    for (int i = 0; i < n; ++i) {
+        const int64_t t = t0 + i;
+        __syncthreads();
+        for (int k = threadIdx.x; k < n_state; k += NVA_WAVE) {
+            b_s[k] = to_float(b_col[t * channels + k]);
+            c_s[k] = to_float(c_col[t * channels + k]);
+        }
+        __syncthreads();
+        if (mode == 2) {
+            float acc = 0.f;
+#pragma unroll
+            for (int k = 0; k < NMAX; ++k)
+                if (k < n_state) acc += S[k] * c_s[k];
+            if (mine) y[t * inner + h * vdim + p] += expf(cum[t * heads + h]) * acc;
+            continue;
+        }
+        const float dt = ssd_softplus(to_float(proj[t * stride + dt_col + h]) + bias);
+        const float decay = expf(rate * dt);
+        const float x = mine ? to_float(conv[t * channels + h * vdim + p]) : 0.f;
+        const float dx = dt * x;
+        float acc = 0.f;
+#pragma unroll
+        for (int k = 0; k < NMAX; ++k) {
+            if (k < n_state) {
+                S[k] = decay * S[k] + b_s[k] * dx;
+                acc += S[k] * c_s[k];
+            }
+        }
+        if (mine) y[t * inner + h * vdim + p] = acc + skip * x;
+        if (mode == 1) {
+            log_decay += rate * dt;
+            if (threadIdx.x == 0 && blockIdx.x == 0) cum[t * heads + h] = log_decay;
+        }
+    }
+    if (mode == 2 || !mine) return;
+    // (a portion of one block has no pass over its blocks: its end state is the request's new state)
+    float* dst = mode == 1 && units[4 * u + 3] > 1 ? block : own;
+#pragma unroll
+    for (int i = 0; i < NMAX; ++i)
+        if (i < n_state) dst[(int64_t)i * vdim] = S[i];
+}
+
+// The pass over a portion's blocks: block_states[b] <- exp(total log-decay of block b) * block_states[b - 1]
+// + block_states[b] for b = 1 ..., and the request's state <- the last.  chains[c] = (first unit, blocks,
+// request, tokens of the last block).  A thread per entry of S.
+__global__ void __launch_bounds__(256)
+ssd_chain_kernel(float* __restrict__ block_states, const float* __restrict__ cum, float* __restrict__ state,
+                 const int32_t* __restrict__ chains, const int32_t* __restrict__ units,
+                 const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, int first_seq, int heads,
+                 int n_state, int vdim) {
+    const int c = blockIdx.z, h = blockIdx.y;
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    const int per_head = n_state * vdim;
+    if (e >= per_head) return;
+    const int u0 = chains[4 * c], blocks = chains[4 * c + 1], s = first_seq + chains[4 * c + 2];
+    const int64_t unit_stride = (int64_t)heads * per_head;
+    float* at = block_states + (int64_t)u0 * unit_stride + (int64_t)h * per_head + e;
+    float carry = at[0];
+    for (int b = 1; b < blocks; ++b) {
+        const int u = u0 + b;
+        const int64_t last = cu_seqlens[first_seq + units[4 * u]] + units[4 * u + 1] + units[4 * u + 2] - 1;
+        carry = expf(cum[last * heads + h]) * carry + at[b * unit_stride];
+        at[b * unit_stride] = carry;
+    }
+    state[((int64_t)state_slots[s] * heads + h) * per_head + e] = carry;
+}
+
+// ---------------------------------------------------------------------------- gate and grouped norm
+template <typename T>
+__global__ void __launch_bounds__(256)
+ssd_finish_kernel(const float* __restrict__ y, const T* __restrict__ proj, int64_t stride, const float* __restrict__ weight,
+                  int inner, int group_size, float eps, T* __restrict__ out, int64_t out_stride) {
+    __shared__ float scratch[16];
+    const int64_t t = blockIdx.x;
+    const int g = blockIdx.y;
+    const float* yr = y + t * inner + g * group_size;
+    const T* zr = proj + t * stride + g * group_size;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < group_size; i += blockDim.x) {
+        const float v = yr[i] * ssd_silu(to_float(zr[i]));
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = rsqrtf(ss / (float)group_size + eps);
+    for (int i = threadIdx.x; i < group_size; i += blockDim.x) {
+        const float v = yr[i] * ssd_silu(to_float(zr[i]));
+        out[t * out_stride + g * group_size + i] = from_float<T>(v * scale * weight[g * group_size + i]);
+    }
+}
+
+template <int NMAX>
+static void launch_scan(dim3 grid, hipStream_t stream, const elem_t* proj, int64_t stride, int dt_col, const elem_t* conv,
+                        int channels, int heads, int vdim, int n_state, int groups, const float* dt_bias, const float* a_log,
+                        const float* d_skip, float* state, const int32_t* cu, const int32_t* starts, const int32_t* slots,
+                        int first_seq, const int32_t* units, int mode, float* block_states, float* cum, float* y) {
+    hipLaunchKernelGGL((ssd_scan_kernel<elem_t, NMAX>), grid, dim3(NVA_WAVE), 0, stream, proj, stride, dt_col, conv, channels,
+                       heads, vdim, n_state, groups, dt_bias, a_log, d_skip, state, cu, starts, slots, first_seq, units, mode,
+                       block_states, cum, y);
+}
+
+// proj: [tokens, 2 H P + 2 G N + H] with rows `stride` apart.  conv_out [tokens, C] (elements), y_raw [tokens, H P]
+// and cum [tokens, H] (float) are scratch.  state [slots, H, N, P], conv_state [slots, C, K - 1], float.
+// The first num_single requests bring one token each.  units / chains (with block_states [units, H, N, P]): the
+// portions of the requests from num_single on cut into blocks (units[u] = request counted from num_single, first token,
+// tokens, blocks of the portion; chains[c] = first unit, blocks, request, tokens of the last block, for every
+// portion of more than one block); null: every portion runs as one.
+NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void* conv_out, float* y_raw, float* cum, void* out,
+                                         int64_t out_stride, float* state, float* conv_state, int64_t slots,
+                                         const int32_t* token_seq, const int32_t* cu_seqlens, const int32_t* seq_starts,
+                                         const int32_t* state_slots, int64_t seqs, int64_t tokens, int64_t num_single,
+                                         int heads, int vdim, int n_state, int groups, int taps, const void* conv_w,
+                                         const void* conv_b, const float* dt_bias, const float* a_log, const float* d_skip,
+                                         const float* norm_w, int norm_groups, float eps, const int32_t* units,
+                                         int64_t n_units, const int32_t* chains, int64_t n_chains, float* block_states,
+                                         hipStream_t stream) {
+    if (tokens == 0) return 0;
+    if (tokens < 0 || seqs <= 0 || seqs > 65535 || num_single < 0 || num_single > seqs || slots <= 0)
+        return nva_fail("state_space: bad counts tokens=%lld requests=%lld", (long long)tokens, (long long)seqs);
+    if (heads <= 0 || vdim <= 0 || n_state <= 0 || groups <= 0 || heads % groups || norm_groups <= 0 ||
+        (heads * vdim) % norm_groups || heads > 65535)
+        return nva_fail("state_space: bad sizes heads=%d vdim=%d state=%d groups=%d norm_groups=%d", heads, vdim, n_state,
+                        groups, norm_groups);
+    if (taps < 1 || taps > SSD_MAX_TAPS) return nva_fail("state_space: %d taps (1..%d are built)", taps, SSD_MAX_TAPS);
+    if (n_state > 256) return nva_fail("state_space: a state of %d rows (up to 256 are built)", n_state);
+    const int inner = heads * vdim, channels = inner + 2 * groups * n_state;
+    if (stride < 2 * inner + 2 * groups * n_state + heads) return nva_fail("state_space: rows too short");
+    if (!proj || !conv_out || !y_raw || !out || !state || !conv_state || !token_seq || !cu_seqlens || !seq_starts ||
+        !state_slots || !conv_w || !conv_b || !dt_bias || !a_log || !d_skip || !norm_w)
+        return nva_fail("state_space: a tensor is missing");
+    if (n_chains && (!units || !chains || !block_states || !cum)) return nva_fail("state_space: blocks need their scratch");
+    const elem_t* pj = (const elem_t*)proj;
+    if (tokens > 0x7fffffff || (channels + 255) / 256 > 65535) return nva_fail("state_space: too many tokens or channels");
+    hipLaunchKernelGGL((ssd_conv_kernel<elem_t>), dim3((unsigned)tokens, (channels + 255) / 256), dim3(256), 0, stream, pj,
+                       stride, inner, channels, taps, (const elem_t*)conv_w, (const elem_t*)conv_b, conv_state, token_seq,
+                       cu_seqlens, seq_starts, state_slots, (elem_t*)conv_out);
+    if (seqs > num_single && taps > 1)
+        hipLaunchKernelGGL((ssd_conv_state_kernel<elem_t>), dim3((channels + 255) / 256, (unsigned)(seqs - num_single)),
+                           dim3(256), 0, stream, pj, stride, inner, channels, taps, conv_state, cu_seqlens, seq_starts,
+                           state_slots, (int)num_single);
+    const int dt_col = inner + channels;
+    auto scan = [&](dim3 grid, int first_seq, const int32_t* us, int mode) {
+        if (n_state <= 16)
+            launch_scan<16>(grid, stream, pj, stride, dt_col, (const elem_t*)conv_out, channels, heads, vdim, n_state, groups,
+                            dt_bias, a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, first_seq, us, mode,
+                            block_states, cum, y_raw);
+        else if (n_state <= 32)
+            launch_scan<32>(grid, stream, pj, stride, dt_col, (const elem_t*)conv_out, channels, heads, vdim, n_state, groups,
+                            dt_bias, a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, first_seq, us, mode,
+                            block_states, cum, y_raw);
+        else if (n_state <= 64)
+            launch_scan<64>(grid, stream, pj, stride, dt_col, (const elem_t*)conv_out, channels, heads, vdim, n_state, groups,
+                            dt_bias, a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, first_seq, us, mode,
+                            block_states, cum, y_raw);
+        else if (n_state <= 128)
+            launch_scan<128>(grid, stream, pj, stride, dt_col, (const elem_t*)conv_out, channels, heads, vdim, n_state, groups,
+                             dt_bias, a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, first_seq, us, mode,
+                             block_states, cum, y_raw);
+        else
+            launch_scan<256>(grid, stream, pj, stride, dt_col, (const elem_t*)conv_out, channels, heads, vdim, n_state, groups,
+                             dt_bias, a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, first_seq, us, mode,
+                             block_states, cum, y_raw);
+    };
+    const unsigned px = (unsigned)((vdim + NVA_WAVE - 1) / NVA_WAVE);
+    if (n_chains) {
+        if (n_units <= 0 || n_units > 65535) return nva_fail("state_space: bad block count %lld", (long long)n_units);
+        if (num_single) scan(dim3(px, heads, (unsigned)num_single), 0, nullptr, 0);
+        scan(dim3(px, heads, (unsigned)n_units), (int)num_single, units, 1);
+        hipLaunchKernelGGL(ssd_chain_kernel, dim3((n_state * vdim + 255) / 256, heads, (unsigned)n_chains), dim3(256), 0, stream,
+                           block_states, cum, state, chains, units, cu_seqlens, state_slots, (int)num_single, heads, n_state,
+                           vdim);
+        scan(dim3(px, heads, (unsigned)n_units), (int)num_single, units, 2);
+    } else {
+        scan(dim3(px, heads, (unsigned)seqs), 0, nullptr, 0);
+    }
+    const int group_size = inner / norm_groups;
+    hipLaunchKernelGGL((ssd_finish_kernel<elem_t>), dim3((unsigned)tokens, norm_groups), dim3(256), 0, stream, y_raw, pj,
+                       stride, norm_w, inner, group_size, eps, (elem_t*)out, out_stride);
+    return nva_check_launch("state_space");
+}
+
+NVA_DEFINE_LAST_ERROR(nva_ssd)

@@ -38,6 +38,8 @@ MODULES: Dict[str, Tuple[str, Tuple[Optional[str], ...]]] = {
     "sample": ("sample.hip", (None,)),
     "qk_rownorm": ("qk_rownorm.hip", ("bf16", "f32")),
     "retention": ("retention.hip", ("bf16", "f32")),
+    "ssd": ("ssd.hip", ("bf16", "f32")),
+    "moe": ("moe.hip", ("bf16", "f32")),
 }
 
 _HEADERS = ("common.h",)

@@ -24,6 +24,7 @@ _LAST_ERROR_SYMBOL = {
     "gemm_skinny": "nva_gemm_skinny_last_error", "gemm_team": "nva_gemm_team_last_error",
     "attn_prefill": "nva_attn_prefill_last_error", "gemm_tile": "nva_gemm_tile_last_error",
     "qk_rownorm": "nva_qk_rownorm_last_error", "retention": "nva_retention_last_error",
+    "ssd": "nva_ssd_last_error", "moe": "nva_moe_last_error",
 }
 
 _loaded: Dict[Tuple[str, Optional[str]], ctypes.CDLL] = {}

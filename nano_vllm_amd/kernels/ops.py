@@ -282,6 +282,8 @@ class HipKernels:
         self.retention_blocks_side_by_side = True
         # False: the general kernel runs one wave per token for portions of prompts too (the same bits, slower)
         self.tiled_general_attention = True
+        # False: the state-space layer runs a portion's tokens one after the other, whatever its length
+        self.state_space_blocks_side_by_side = True
 
     # ------------------------------------------------------------------ helpers
     def _stream(self):
@@ -435,8 +437,152 @@ class HipKernels:
                      self._stream())
         return out, residual
 
+    def stream_dyt(self, addends, residual: Optional[torch.Tensor], weight: torch.Tensor, bias: torch.Tensor,
+                   alpha: torch.Tensor, out: Optional[torch.Tensor] = None):
+        """The Dynamic Tanh norm of a residual stream kept in float32: residual <- residual + sum(addends) in
+        place (residual None: a new stream that starts as the sum), then y = tanh(alpha * residual) * weight +
+        bias, all float, rounded once.  addends: one or two tensors of the element type [rows, width]; weight
+        and bias float32 [width], alpha a float32 tensor of one number (read on the device).  Returns
+        (y, residual)."""
+        addends = [_t(a) for a in addends]
+        if not 1 <= len(addends) <= 2:
+            raise KernelError("stream_dyt: one or two addends")
+        ref = addends[0]
+        rows, width = ref.shape
+        args = []
+        for a in addends:
+            if tuple(a.shape) != (rows, width) or a.dtype != ref.dtype:
+                raise KernelError("stream_dyt: the addends differ in shape or type")
+            _, _, as_ = _rows2d(a, "stream_dyt addend")
+            args += [_p(a), c_i64(as_)]
+        if len(addends) == 1:
+            args += [None, c_i64(0)]
+        first = residual is None
+        if first:
+            residual = torch.empty((rows, width), dtype=torch.float32, device=ref.device)
+        rrows, rw, rs = _rows2d(residual, "stream_dyt residual")
+        if (rrows, rw) != (rows, width) or residual.dtype != torch.float32:
+            raise KernelError("stream_dyt: the residual stream must be float32 of the addends' shape")
+        for v, what in ((weight, "weight"), (bias, "bias")):
+            if v.dtype != torch.float32 or tuple(v.shape) != (width,) or not v.is_contiguous():
+                raise KernelError(f"stream_dyt: {what} must be contiguous float32 [{width}]")
+        if alpha.dtype != torch.float32 or alpha.numel() != 1:
+            raise KernelError("stream_dyt: alpha must be one float32 number")
+        if out is None:
+            out = torch.empty((rows, width), dtype=ref.dtype, device=ref.device)
+        orows, ow, os_ = _rows2d(out, "stream_dyt output")
+        if (orows, ow) != (rows, width) or out.dtype != ref.dtype:
+            raise KernelError("stream_dyt: output does not match")
+        library.call("norm", _suffix(out), "nva_stream_dyt", *args, _p(residual), c_i64(rs), c_i32(1 if first else 0),
+                     _p(weight), _p(bias), _p(alpha), _p(out), c_i64(os_), c_i64(rows), c_i32(width), self._stream())
+        return out, residual
+
+    def pair_norm_mean(self, a, wa: torch.Tensor, b, wb: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None):
+        """(a * rsqrt(mean(a^2) + eps) * wa + b * rsqrt(mean(b^2) + eps) * wb) / 2 over rows of the model width;
+        wa, wb float32 [width].  An input left as a split product's partial sums is added up while it is read."""
+        a, b = [x if isinstance(x, SplitSum) and self.fuse_split_sums else _t(x) for x in (a, b)]
+        rows, width = a.shape
+        if tuple(b.shape) != (rows, width) or a.dtype != b.dtype:
+            raise KernelError("pair_norm_mean: the inputs differ in shape or type")
+        for w in (wa, wb):
+            if w.dtype != torch.float32 or tuple(w.shape) != (width,) or not w.is_contiguous():
+                raise KernelError(f"pair_norm_mean: the weights must be contiguous float32 [{width}]")
+        args = []
+        for x, w in ((a, wa), (b, wb)):
+            if isinstance(x, SplitSum):
+                args += [None, c_i64(0), _p(x.sums), c_i32(x.splits), c_i64(rows * width), _p(x.bias), _p(w)]
+            else:
+                _, _, xs = _rows2d(x, "pair_norm_mean input")
+                args += [_p(x), c_i64(xs), None, c_i32(0), c_i64(0), None, _p(w)]
+        if out is None:
+            out = torch.empty((rows, width), dtype=a.dtype, device=a.device)
+        orows, ow, os_ = _rows2d(out, "pair_norm_mean output")
+        if (orows, ow) != (rows, width) or out.dtype != a.dtype:
+            raise KernelError("pair_norm_mean: output does not match")
+        library.call("norm", _suffix(out), "nva_pair_norm_mean", *args, _p(out), c_i64(os_), c_i64(rows), c_i32(width),
+                     c_f32(eps), self._stream())
+        return out
+
+    def scale_(self, x: torch.Tensor, factor: float) -> torch.Tensor:
+        """x <- x * factor in place; x float32 [rows, width]."""
+        rows, width, xs = _rows2d(x, "scale_ input")
+        if x.dtype != torch.float32:
+            raise KernelError("scale_: the tensor must be float32")
+        library.call("embed", self.suffix, "nva_scale_rows", _p(x), c_i64(xs), c_i64(rows), c_i32(width), c_f32(factor),
+                     self._stream())
+        return x
+
     # ------------------------------------------------------------------ feed-forward
     ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+    PLAIN_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2, "relu2": 3}
+
+    def act(self, x: torch.Tensor, act: str = "relu2", out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """act(x), entry by entry: silu, relu, gelu_tanh or relu2 (the square of relu)."""
+        if act not in self.PLAIN_ACTIVATIONS:
+            raise KernelError(f"act: unknown activation {act!r}; known: {sorted(self.PLAIN_ACTIVATIONS)}")
+        x = _t(x)
+        rows, width, xs = _rows2d(x, "act input")
+        if out is None:
+            out = torch.empty((rows, width), dtype=x.dtype, device=x.device)
+        orows, ow, os_ = _rows2d(out, "act output")
+        if (orows, ow) != (rows, width) or out.dtype != x.dtype:
+            raise KernelError("act: output does not match the input")
+        library.call("activation", _suffix(x), "nva_act", _p(x), c_i64(xs), _p(out), c_i64(os_), c_i64(rows), c_i32(width),
+                     c_i32(self.PLAIN_ACTIVATIONS[act]), self._stream())
+        return out
+
+    # ------------------------------------------------------------------ routed feed-forward
+    def moe_route(self, logits: torch.Tensor, top: int, group_count: int, group_keep: int, scale: float):
+        """From the router's float32 logits [tokens, experts]: int32 [tokens, top] experts and float32
+        [tokens, top] weights (scale * sigmoid score).  Experts form group_count groups of neighbours; a
+        group's score is the sum of its two largest scores; only experts of the group_keep best groups are
+        chosen, the `top` with the largest scores."""
+        rows, experts, ls = _rows2d(logits, "router logits")
+        if logits.dtype != torch.float32:
+            raise KernelError("moe_route: the logits must be float32")
+        ids = torch.empty((rows, top), dtype=torch.int32, device=logits.device)
+        weights = torch.empty((rows, top), dtype=torch.float32, device=logits.device)
+        library.call("moe", self.suffix, "nva_moe_route", _p(logits), c_i64(ls), c_i64(rows), c_i32(experts), c_i32(top),
+                     c_i32(group_count), c_i32(group_keep), c_f32(scale), _p(ids), _p(weights), self._stream())
+        return ids, weights
+
+    def moe_experts(self, x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, up: torch.Tensor, down: torch.Tensor,
+                    num_experts: int, act: str = "relu2", add=None) -> torch.Tensor:
+        """y[t] = sum over the choices c of weights[t, c] * act(x[t] Wu_e^T) Wd_e^T with e = ids[t, c] (+ add[t]).
+        up [E * ff, k] and down [E * k, ff] hold the experts' matrices one below the other."""
+        if act not in self.PLAIN_ACTIVATIONS:
+            raise KernelError(f"moe_experts: unknown activation {act!r}")
+        x = _t(x)
+        tokens, k, xs = _rows2d(x, "moe input")
+        if up.dim() != 2 or down.dim() != 2 or up.shape[0] % num_experts or up.shape[1] != k or not up.is_contiguous() \
+                or not down.is_contiguous() or up.dtype != x.dtype or down.dtype != x.dtype:
+            raise KernelError("moe_experts: the experts' matrices do not fit the input")
+        ff = up.shape[0] // num_experts
+        if tuple(down.shape) != (num_experts * k, ff):
+            raise KernelError(f"moe_experts: down must be [{num_experts * k}, {ff}], got {tuple(down.shape)}")
+        top = ids.shape[1] if ids.dim() == 2 else 0
+        if ids.dtype != torch.int32 or tuple(ids.shape) != (tokens, top) or not ids.is_contiguous() or top <= 0 or \
+                weights.dtype != torch.float32 or tuple(weights.shape) != (tokens, top) or not weights.is_contiguous():
+            raise KernelError("moe_experts: ids int32 and weights float32, both contiguous [tokens, top]")
+        add_stride = 0
+        if add is not None:
+            add = _t(add)
+            arows, aw, add_stride = _rows2d(add, "moe addend")
+            if (arows, aw) != (tokens, k) or add.dtype != x.dtype:
+                raise KernelError("moe_experts: the addend does not match the input")
+        pairs = tokens * top
+        tile_rows = library.load("moe", self.suffix)
+        bm = int(getattr(tile_rows, f"nva_moe_tile_rows_{self.suffix}")())
+        max_tiles = pairs // bm + num_experts
+        ints = torch.empty(2 * pairs + 3 * max_tiles + 1, dtype=torch.int32, device=x.device)
+        hidden = torch.empty((pairs, ff), dtype=x.dtype, device=x.device)
+        outs = torch.empty((pairs, k), dtype=x.dtype, device=x.device)
+        y = torch.empty((tokens, k), dtype=x.dtype, device=x.device)
+        library.call("moe", _suffix(x), "nva_moe_experts", _p(x), c_i64(xs), _p(ids), _p(weights), c_i64(tokens), c_i32(top),
+                     c_i32(num_experts), c_i32(k), c_i32(ff), _p(up), _p(down), c_i32(self.PLAIN_ACTIVATIONS[act]), _p(add),
+                     c_i64(add_stride), _p(ints[:pairs]), _p(ints[pairs:2 * pairs]), _p(ints[2 * pairs:]), c_i64(max_tiles),
+                     _p(hidden), _p(outs), _p(y), c_i64(k), self._stream())
+        return y
 
     def act_mul(self, gate_up: torch.Tensor, act: str = "silu", out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """act(gate) * up of a row [gate | up]; act: silu, relu or gelu_tanh."""
@@ -845,6 +991,19 @@ class HipKernels:
                      self._stream())
         return table
 
+    def rotary_step_table(self, inv_freq: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        """float32 [tokens, 2 * len(inv_freq)]: cos(p_t * f), then sin(p_t * f), for the step's tokens at their
+        positions p_t (int32, read on the device)."""
+        if inv_freq.dtype != torch.float32 or inv_freq.dim() != 1 or not inv_freq.is_contiguous():
+            raise KernelError("rotary_step_table: inv_freq must be contiguous float32")
+        tokens = positions.shape[0]
+        _i32(positions, tokens, "positions")
+        half = inv_freq.shape[0]
+        table = torch.empty((tokens, 2 * half), dtype=torch.float32, device=inv_freq.device)
+        library.call("rope", self.suffix, "nva_rotary_step_table", _p(inv_freq), c_i32(half), _p(positions), c_i64(tokens),
+                     _p(table), self._stream())
+        return table
+
     def qk_norm_rope_store(self, qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                            q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                            table: Optional[torch.Tensor], positions: Optional[torch.Tensor],
@@ -915,8 +1074,10 @@ class HipKernels:
                          q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                          positions: Optional[torch.Tensor], temp_coef: float, temp_every: int,
                          slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
-                         v_cache: Optional[torch.Tensor]) -> torch.Tensor:
-        """q and k normed over the whole projection (all heads at once, plain weights [heads * head_dim]
+                         v_cache: Optional[torch.Tensor], rot_table: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """rot_table, float32 [tokens, rot]: after norm and temperature the first rot channels of every head
+        of q and k are rotated in pairs (i, i + rot / 2) by the token's row (rot / 2 cosines, then sines).
+        q and k normed over the whole projection (all heads at once, plain weights [heads * head_dim]
         and [kv_heads * head_dim]), q scaled by the temperature 1 + temp_coef * ln(floor((p + 1) /
         temp_every) + 1) of its position p, both written back in place, k and v written into their page
         slots.  The row is [q | k | v] with values of v_head_dim.  Returns the q view."""
@@ -941,6 +1102,13 @@ class HipKernels:
             if positions is None or int(temp_every) <= 0:
                 raise KernelError("a query temperature needs the positions and a positive step")
             _i32(positions, tokens, "positions")
+        rot = 0
+        if rot_table is not None:
+            rot = rot_table.shape[1] if rot_table.dim() == 2 else 0
+            if rot_table.dtype != torch.float32 or rot_table.dim() != 2 or rot_table.shape[0] != tokens or \
+                    not rot_table.is_contiguous() or rot <= 0 or rot % 2 or rot > head_dim:
+                raise KernelError(f"qk_rownorm_store: the rotation table must be contiguous float32 [{tokens}, rot], rot "
+                                  f"even and at most the head's {head_dim}")
         page_size = 0
         if k_cache is not None:
             page_size = self._check_cache(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype, v_head_dim)
@@ -956,7 +1124,7 @@ class HipKernels:
         library.call("qk_rownorm", "bf16" if partial else _suffix(qkv), "nva_qk_rownorm_store", *source, c_i64(tokens),
                      c_i32(num_heads), c_i32(num_kv_heads), c_i32(head_dim), c_i32(v_head_dim), _p(q_weight), _p(k_weight),
                      c_i32(wf), c_f32(eps), _p(positions), c_f32(float(temp_coef)), c_i32(int(temp_every) if temp_coef else 1),
-                     _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size), self._stream())
+                     _p(rot_table), c_i32(rot), _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size), self._stream())
         return q
 
     @staticmethod
@@ -977,8 +1145,10 @@ class HipKernels:
     def paged_attention(self, q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                         k_cache: torch.Tensor, v_cache: torch.Tensor, batch, group: int, scale: float,
                         window: Optional[int] = None, out: Optional[torch.Tensor] = None,
-                        v_head_dim: Optional[int] = None, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Causal attention of the step's tokens over the cache.  `batch` is the step's
+                        v_head_dim: Optional[int] = None, sinks: Optional[torch.Tensor] = None,
+                        chunk: Optional[int] = None) -> torch.Tensor:
+        """chunk: a query at position p reads the keys from floor(p / chunk) * chunk on only.
+        Causal attention of the step's tokens over the cache.  `batch` is the step's
         StepBatch; `group` selects its block tables.  q [T, heads*head_dim] (rows may be strided).
         v_head_dim: the size of a head's values where it is not head_dim (the output is then
         [T, heads*v_head_dim]).  sinks, float32 [heads]: one more term exp(sink_h) in the denominator
@@ -1012,7 +1182,8 @@ class HipKernels:
         # them where its shape limits allow; everything else runs the general kernel
         start = 0
         # (the matrix-core kernels fold the scale into the exponent, which needs it positive)
-        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim
+        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim \
+            and not chunk
         if batch.num_decode > 0 and mfma and \
                 self._decode_kernel_takes(num_heads // num_kv_heads, head_dim, page_size, q, qs, out, os_):
             start = batch.num_decode
@@ -1036,8 +1207,8 @@ class HipKernels:
             library.call("attn_generic", _suffix(q), "nva_paged_attention_tiled", _p(q), c_i64(qs), _p(out), c_i64(os_),
                          _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.cu_seqlens_q),
                          _p(batch.kv_lens), _p(tiles), c_i64(tiles.shape[0]), c_i32(num_heads), c_i32(num_kv_heads),
-                         c_i32(head_dim), c_i32(v_dim), c_i32(page_size), c_f32(scale), _p(sinks), _p(self.fault_flag),
-                         self._stream())
+                         c_i32(head_dim), c_i32(v_dim), c_i32(page_size), c_f32(scale), c_i32(chunk or 0), _p(sinks),
+                         _p(self.fault_flag), self._stream())
             tokens = batch.num_decode            # what is left: the single tokens before the portions
         if start < tokens:
             n = tokens - start
@@ -1045,7 +1216,78 @@ class HipKernels:
                          _p(out[start:]), c_i64(os_), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
                          _p(batch.token_seq[start:]), _p(batch.positions[start:]), c_i64(n), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(v_dim), c_i32(page_size), c_f32(scale),
-                         c_i32(window or 0), _p(sinks), _p(self.fault_flag), self._stream())
+                         c_i32(window or 0), c_i32(chunk or 0), _p(sinks), _p(self.fault_flag), self._stream())
+        return out
+
+    # ------------------------------------------------------------------ state-space layer
+    def state_space(self, proj: torch.Tensor, heads: int, vdim: int, n_state: int, groups: int, taps: int,
+                    conv_w: torch.Tensor, conv_b: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor,
+                    d_skip: torch.Tensor, norm_w: torch.Tensor, norm_groups: int, eps: float, conv_state: torch.Tensor,
+                    ssm_state: torch.Tensor, batch, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """A selective state-space layer over the step's tokens: proj [T, 2 H P + 2 G N + H] = [z | x B C | dt].
+        x, B, C pass a causal convolution of `taps` taps per channel (conv_w [C, taps], conv_b [C]) and silu;
+        dt <- softplus(dt + dt_bias); per head S <- exp(-exp(a_log) dt) S + dt B x^T, y = S^T C + d_skip x; then
+        y * silu(z), an RMS norm in norm_groups parts, times norm_w.  ssm_state float32 [slots, H, N, P] and
+        conv_state float32 [slots, C, taps - 1] hold a request's state in the row batch.state_slots names, taken
+        as zero where batch.seq_starts is 0.  Returns [T, H P] of proj's type."""
+        proj = _t(proj)
+        tokens, width, stride = _rows2d(proj, "state-space projections")
+        inner, gn = heads * vdim, groups * n_state
+        channels = inner + 2 * gn
+        if width != 2 * inner + 2 * gn + heads:
+            raise KernelError(f"state_space: projections of width {width}, expected {2 * inner + 2 * gn + heads}")
+        if ssm_state.dtype != torch.float32 or tuple(ssm_state.shape[1:]) != (heads, n_state, vdim) or not ssm_state.is_contiguous():
+            raise KernelError(f"state_space: the state must be contiguous float32 [slots, {heads}, {n_state}, {vdim}]")
+        if conv_state.dtype != torch.float32 or tuple(conv_state.shape) != (ssm_state.shape[0], channels, taps - 1) or \
+                not conv_state.is_contiguous():
+            raise KernelError(f"state_space: the kept inputs must be contiguous float32 [slots, {channels}, {taps - 1}]")
+        if tuple(conv_w.shape) != (channels, taps) or tuple(conv_b.shape) != (channels,) or conv_w.dtype != proj.dtype or \
+                conv_b.dtype != proj.dtype or not conv_w.is_contiguous() or not conv_b.is_contiguous():
+            raise KernelError("state_space: the convolution's weights do not fit")
+        for v, n, what in ((dt_bias, heads, "dt_bias"), (a_log, heads, "a_log"), (d_skip, heads, "d_skip"), (norm_w, inner, "norm_w")):
+            if v.dtype != torch.float32 or tuple(v.shape) != (n,) or not v.is_contiguous():
+                raise KernelError(f"state_space: {what} must be contiguous float32 [{n}]")
+        seqs = batch.num_seqs
+        _i32(batch.token_seq, tokens, "token_seq")
+        _i32(batch.cu_seqlens_q, seqs + 1, "cu_seqlens_q")
+        _i32(batch.seq_starts, seqs, "seq_starts")
+        _i32(batch.state_slots, seqs, "state_slots")
+        if sum(batch.q_lens) != tokens or any(n != 1 for n in batch.q_lens[:batch.num_decode]):
+            raise KernelError("state_space: the batch does not describe the projections' rows (single tokens first)")
+        if out is None:
+            out = torch.empty((tokens, inner), dtype=proj.dtype, device=proj.device)
+        orows, ow, os_ = _rows2d(out, "state-space output")
+        if (orows, ow) != (tokens, inner) or out.dtype != proj.dtype:
+            raise KernelError("state_space: output does not match")
+        conv_out = torch.empty((tokens, channels), dtype=proj.dtype, device=proj.device)
+        y_raw = torch.empty((tokens, inner), dtype=torch.float32, device=proj.device)
+        # long portions are cut into blocks that run side by side (the same cut for every layer of the step)
+        units = chains = block_states = cum = None
+        n_units = n_chains = 0
+        first = batch.num_decode
+        if self.state_space_blocks_side_by_side and first < seqs:
+            kept = getattr(batch, "step_cache", None)
+            if kept is None:
+                kept = batch.step_cache = {}
+            plan = kept.get(("state_space_blocks", first))
+            if plan is None:
+                _, flat_units, flat_chains = retention_blocks(batch.q_lens, first)
+                if flat_chains:
+                    both = torch.tensor(flat_units + flat_chains, dtype=torch.int32).to(proj.device, non_blocking=True)
+                    plan = (len(flat_units) // 4, len(flat_chains) // 4, both[: len(flat_units)], both[len(flat_units):])
+                else:
+                    plan = (0, 0, None, None)
+                kept[("state_space_blocks", first)] = plan
+            n_units, n_chains, units, chains = plan
+            if n_chains:
+                block_states = torch.empty((n_units, heads, n_state, vdim), dtype=torch.float32, device=proj.device)
+                cum = torch.empty((tokens, heads), dtype=torch.float32, device=proj.device)
+        library.call("ssd", _suffix(proj), "nva_state_space", _p(proj), c_i64(stride), _p(conv_out), _p(y_raw), _p(cum), _p(out),
+                     c_i64(os_), _p(ssm_state), _p(conv_state), c_i64(ssm_state.shape[0]), _p(batch.token_seq),
+                     _p(batch.cu_seqlens_q), _p(batch.seq_starts), _p(batch.state_slots), c_i64(seqs), c_i64(tokens),
+                     c_i64(first), c_i32(heads), c_i32(vdim), c_i32(n_state), c_i32(groups), c_i32(taps), _p(conv_w),
+                     _p(conv_b), _p(dt_bias), _p(a_log), _p(d_skip), _p(norm_w), c_i32(norm_groups), c_f32(eps), _p(units),
+                     c_i64(n_units), _p(chains), c_i64(n_chains), _p(block_states), self._stream())
         return out
 
     # ------------------------------------------------------------------ retention
