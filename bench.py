@@ -24,6 +24,12 @@ is another measurement and leaves the default one as it is: prefill and decode t
 Nozurax design (alternating attention and retention layers) beside a Qwen3 model of the same layer
 sizes, a few layers of each with random weights, through the same step function; one JSON line
 with both designs' numbers per size.
+
+    python bench.py --design mafarax [--design-sizes 1024,2048,4096] [--layers 4]
+
+does the same for the Mafarax design (every layer a chunked attention and a state-space layer side by
+side, and a routed feed-forward whose experts a token runs add up to the dense layer's inner size),
+beside Nozurax and Qwen3 at equal layer sizes.
 """
 import argparse
 import json
@@ -55,7 +61,7 @@ def parse_args():
                     help="context of one more decode point at the default batch (0: none)")
     ap.add_argument("--serve-seqs", type=int, default=256,
                     help="requests of the reference's benchmark workload through LLM.generate (0: not run)")
-    ap.add_argument("--design", default=None, choices=["nozurax"],
+    ap.add_argument("--design", default=None, choices=["nozurax", "mafarax"],
                     help="measure this design beside Qwen3 at equal layer sizes instead of the default workload")
     ap.add_argument("--design-sizes", default="1024,2048,4096", help="model widths of the --design measurement")
     return ap.parse_args()
@@ -67,8 +73,27 @@ DESIGN_SIZES = {1024: (16, 8, 128, 3072), 2048: (16, 8, 128, 6144), 4096: (32, 8
 DESIGN_VOCAB = 32768
 
 
-def design_configs(width: int, layers: int, dtype: str):
-    """config.json of a Nozurax model and of the Qwen3 model with the same layer sizes."""
+def mafarax_config(width: int, layers: int, dtype: str) -> dict:
+    """A Mafarax model of the width's layer sizes: the attention half with the dense model's heads (equal key and
+    value sizes, chunks of 1024 positions, half the head rotated), the state-space half with twice the width in
+    heads of 64 channels and 128 state rows, 32 experts of an eighth of the dense inner size of which a token
+    runs 6, chosen among 4 of 8 groups, and a shared expert of a quarter of it."""
+    heads, kv, dim, inner = DESIGN_SIZES[width]
+    layer = {"type": "parallel",
+             "mixer": {"left": {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                "mask": {"size": 1024}, "rot": {"dims": dim // 2, "base": 5e5, "scaling": {"factor": 2.0}}},
+                       "right": {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 1}},
+             "mlp": {"kind": "moe", "expert": {"ff": inner // 8}, "shared": {"ff": inner // 4},
+                     "router": {"experts": 32, "top": 6, "scale": 1.0, "groups": {"count": 8, "keep": 4}}}}
+    return {"architecture": "Mafarax", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+            "layers": [layer] * layers, "torch_dtype": dtype}
+
+
+def design_configs(width: int, layers: int, dtype: str, design: str = "nozurax"):
+    """config.json of a Nozurax model and of the Qwen3 model with the same layer sizes (and, for the Mafarax
+    measurement, of the Mafarax model first)."""
+    if design == "mafarax":
+        return {"mafarax": mafarax_config(width, layers, dtype), **design_configs(width, layers, dtype)}
     heads, kv, dim, inner = DESIGN_SIZES[width]
     att = {"type": "attention", "mlp": {"kind": "dense", "ff": inner},
            "mixer": {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
@@ -102,7 +127,7 @@ def design_run(args):
     out = {}
     for width in [int(w) for w in args.design_sizes.split(",") if w]:
         out[width] = {}
-        for name, config_json in design_configs(width, layers, args.dtype).items():
+        for name, config_json in design_configs(width, layers, args.dtype, args.design).items():
             arch = architecture_of(config_json)
             model = Model(arch.build_spec(arch.parse_config(config_json)), kernels, device, dtype)
             fill_random_(model, args.seed)
@@ -157,11 +182,11 @@ def design_run(args):
             torch.cuda.empty_cache()
     first = out[next(iter(out))]
     line = {"metric": f"--design {args.design}: prefill tok/s @ {T} tokens and decode tok/s @ batch {B}, context {ctx}, "
-                      f"{layers} layers, beside Qwen3 at equal layer sizes",
+                      f"{layers} layers, beside {'Nozurax and ' if args.design == 'mafarax' else ''}Qwen3 at equal layer sizes",
             "value": first[args.design]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": first[args.design]["decode_ms_per_step"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-            "data": "synthetic", "config": {"model": f"{args.design} and qwen3, random weights", "global_batch": B,
+            "data": "synthetic", "config": {"model": f"{', '.join(first)}, random weights", "global_batch": B,
                                             "seq_len": ctx, "parallelism": "single GPU", "layers": layers,
                                             "vocab_size": DESIGN_VOCAB, "decode_graph": not args.eager},
             "designs": {str(w): v for w, v in out.items()}}

@@ -280,7 +280,7 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
     if (n_state > 256) return nva_fail("state_space: a state of %d rows (up to 256 are built)", n_state);
     const int inner = heads * vdim, channels = inner + 2 * groups * n_state;
     if (stride < 2 * inner + 2 * groups * n_state + heads) return nva_fail("state_space: rows too short");
-    if (!proj || !conv_out || !y_raw || !out || !state || !conv_state || !token_seq || !cu_seqlens || !seq_starts ||
+    if (!proj || !conv_out || !y_raw || !out || !state || (!conv_state && taps > 1) || !token_seq || !cu_seqlens || !seq_starts ||
         !state_slots || !conv_w || !conv_b || !dt_bias || !a_log || !d_skip || !norm_w)
         return nva_fail("state_space: a tensor is missing");
     if (n_chains && (!units || !chains || !block_states || !cum)) return nva_fail("state_space: blocks need their scratch");
