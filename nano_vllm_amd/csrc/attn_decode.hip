@@ -2,7 +2,8 @@
 // request's keys in the paged cache, split over the context.
 //
 // Semantics as in attn_generic.hip (nanovllm/layers/attention.py:71-74, causal).  The token at
-// position p reads keys first..p, first = max(0, p - window + 1) with a window, else 0.
+// position p reads keys first..p, first = max(0, p - window + 1) with a window, the start of p's chunk of positions
+// with chunks (nva_first_key), else 0.
 //
 // Work split: the keys that the step's tokens see are cut into equal quotas, one per wave and kv
 // head (see the plan below).  The G = Hq / Hkv query heads of a kv head share its keys: they are
@@ -102,7 +103,7 @@ __host__ __device__ inline int decode_quota_cap(int page_size) {
 
 __global__ void __launch_bounds__(NVA_WAVE)
 attn_decode_plan_kernel(const int32_t* __restrict__ positions, const int32_t* __restrict__ token_seq, int tokens,
-                        int page_size, int window, int max_segments, int waves_per_head, int32_t* __restrict__ plan,
+                        int page_size, int window, int chunk, int max_segments, int waves_per_head, int32_t* __restrict__ plan,
                         int32_t* error_flag) {
     const int lane = threadIdx.x;
     // every lane's tokens: position (-1: no such token) and the chunks it sees
@@ -116,7 +117,7 @@ attn_decode_plan_kernel(const int32_t* __restrict__ positions, const int32_t* __
 #pragma unroll
     for (int i = 0; i < DEC_MAX_TOKENS / NVA_WAVE; ++i)
         if (pos_r[i] >= 0) {
-            const int first = window > 0 && pos_r[i] - window + 1 > 0 ? pos_r[i] - window + 1 : 0;
+            const int first = nva_first_key(pos_r[i], window, chunk);
             total += pos_r[i] / DEC_CHUNK - first / DEC_CHUNK + 1;
         }
 #pragma unroll
@@ -139,7 +140,7 @@ attn_decode_plan_kernel(const int32_t* __restrict__ positions, const int32_t* __
         if (i * NVA_WAVE >= tokens) break;
         const int t = i * NVA_WAVE + lane;
         const int pos = pos_r[i];
-        const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+        const int first = nva_first_key(pos, window, chunk);
         const int c = pos >= 0 && num_quotas > 0 ? pos / DEC_CHUNK - first / DEC_CHUNK + 1 : 0;
         int incl = c;
 #pragma unroll
@@ -188,7 +189,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
                    float* __restrict__ part_o, float* __restrict__ part_ml, const int32_t* __restrict__ plan,
                    const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
                    const int32_t* __restrict__ block_tables, int table_stride, int tokens, int max_segments,
-                   int num_q_heads, int num_kv_heads, int page_size, float scale, int window,
+                   int num_q_heads, int num_kv_heads, int page_size, float scale, int window, int chunk,
                    const float* __restrict__ sinks, int32_t* error_flag) {
     constexpr int KP = D / 32;          // 16-byte pieces of a key row per lane = MFMAs per S tile
     constexpr int DT = D / 16;          // 16-channel tiles of the output
@@ -210,7 +211,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
 
     // A segment's block table entries: lane i keeps the entry of page lo / page_size + i (a segment
     // spans at most 62 pages, so no chunk needs the table again).
-    auto first_of = [&](const int4& r) { return window > 0 && r.z - window + 1 > 0 ? r.z - window + 1 : 0; };
+    auto first_of = [&](const int4& r) { return nva_first_key(r.z, window, chunk); };
     auto window_of = [&](const int4& r, int lo) {
         const int page0 = lo / page_size;
         return page0 + lane <= r.z / page_size ? block_tables[(int64_t)r.y * table_stride + page0 + lane] : -1;
@@ -579,13 +580,14 @@ NVA_EXPORT int nva_attn_decode_plan_size_bf16(int longest, int64_t tokens, int n
 // Makes the plan of a step (once per step and cache group; every layer's attention reads it).
 // max_segments and waves from nva_attn_decode_plan_size for the same tokens, kv heads and page size.
 NVA_EXPORT int nva_attn_decode_plan_bf16(const int32_t* positions, const int32_t* token_seq, int64_t tokens,
-                                         int num_kv_heads, int page_size, int window, int max_segments, int waves,
-                                         int32_t* plan, int32_t* error_flag, hipStream_t stream) {
+                                         int num_kv_heads, int page_size, int window, int chunk, int max_segments,
+                                         int waves, int32_t* plan, int32_t* error_flag, hipStream_t stream) {
     if (!positions || !token_seq || !plan || !nva_aligned(plan, 16) || tokens <= 0 || tokens > DEC_MAX_TOKENS ||
-        num_kv_heads <= 0 || page_size <= 0 || window < 0 || max_segments <= tokens || waves <= 0 || waves % num_kv_heads)
+        num_kv_heads <= 0 || page_size <= 0 || window < 0 || chunk < 0 || max_segments <= tokens || waves <= 0 ||
+        waves % num_kv_heads)
         return nva_fail("attn_decode_plan: bad arguments");
     hipLaunchKernelGGL(attn_decode_plan_kernel, dim3(1), dim3(NVA_WAVE), 0, stream, positions, token_seq, (int)tokens,
-                       page_size, window, max_segments, waves / num_kv_heads, plan, error_flag);
+                       page_size, window, chunk, max_segments, waves / num_kv_heads, plan, error_flag);
     return nva_check_launch("attn_decode_plan");
 }
 
@@ -596,7 +598,7 @@ NVA_EXPORT int nva_attn_decode_plan_bf16(const int32_t* positions, const int32_t
 NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride, float* scratch,
                                     const int32_t* plan, const void* k_cache, const void* v_cache,
                                     const int32_t* block_tables, int table_stride, int64_t tokens, int num_q_heads,
-                                    int num_kv_heads, int head_dim, int page_size, float scale, int window,
+                                    int num_kv_heads, int head_dim, int page_size, float scale, int window, int chunk,
                                     int max_segments, int waves, const float* sinks, int32_t* error_flag,
                                     hipStream_t stream) {
     if (tokens == 0) return 0;
@@ -616,7 +618,7 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     if (tokens < 0 || tokens > DEC_MAX_TOKENS || num_q_heads > 65535)
         return nva_fail("attn_decode: %lld tokens (at most %d a launch) or %d heads exceed the grid", (long long)tokens,
                         DEC_MAX_TOKENS, num_q_heads);
-    if (max_segments <= tokens || waves <= 0 || waves % num_kv_heads || window < 0 || table_stride <= 0 || !scratch ||
+    if (max_segments <= tokens || waves <= 0 || waves % num_kv_heads || window < 0 || chunk < 0 || table_stride <= 0 || !scratch ||
         !plan || !nva_aligned(plan, 16))
         return nva_fail("attn_decode: bad plan (%d segments, %d waves), window %d or no scratch", max_segments, waves,
                         window);
@@ -626,7 +628,7 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     hipLaunchKernelGGL(attn_decode_kernel<DD>, dim3((unsigned)waves), dim3(NVA_WAVE), 0, stream, (const __bf16*)q, \
                        q_stride, (__bf16*)out, out_stride, part_o, part_ml, plan, (const __bf16*)k_cache,         \
                        (const __bf16*)v_cache, block_tables, table_stride, (int)tokens, max_segments, num_q_heads,  \
-                       num_kv_heads, page_size, scale, window, sinks, error_flag)
+                       num_kv_heads, page_size, scale, window, chunk, sinks, error_flag)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;

@@ -4,7 +4,8 @@
 // aligned to the end of the keys when a request has cached tokens before this step's).  A request
 // with q_len new tokens and kv_len tokens in the cache after this step has its query i at position
 // kv_len - q_len + i; it reads keys first..position, first = max(0, position - window + 1) with a
-// window, else 0.  The step's own keys are in the cache already.
+// window, the start of the position's chunk with chunks (nva_first_key), else 0.  The step's own keys are in
+// the cache already.
 //
 // Work split: a workgroup takes 32 query rows of one request and up to 4 query heads of one kv head
 // (one head per wave), so that a K/V tile is fetched once for the group.  A CU holds 8 of these waves
@@ -93,7 +94,8 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
                     const int32_t* __restrict__ block_tables, int table_stride,
                     const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ kv_lens,
                     const int32_t* __restrict__ tiles, int num_tiles, int paired, int num_q_heads, int num_kv_heads,
-                    int page_size, float scale, int window, const float* __restrict__ sinks, int32_t* error_flag) {
+                    int page_size, float scale, int window, int key_chunk, const float* __restrict__ sinks,
+                    int32_t* error_flag) {
     constexpr int DC = D / 16;            // 16-channel steps of the first product
     constexpr int MT = D / 32;            // 32-channel tiles of the output
     constexpr int KR = D / 8;             // 16-byte pieces of a K row (one key)
@@ -155,7 +157,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
 
     // keys any row of the tile may see
     const int last_pos = start + min(q0 + PF_BM, q_len) - 1;
-    const int first_any = window > 0 && start + q0 - window + 1 > 0 ? start + q0 - window + 1 : 0;
+    const int first_any = nva_first_key(start + q0, window, key_chunk);
     const int kb_lo = first_any & ~(PF_BN - 1);
     const int kb_hi = last_pos + 1;                   // exclusive
 
@@ -184,7 +186,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     // S tile row r = col holds key 16*(a/2) + 8*h' + 4*(a%2) + b with a = r/8, h' = (r/4)%2, b = r%4
     const int a_r = col >> 3, h_r = (col >> 2) & 1, b_r = col & 3;
     const int row_key = 16 * (a_r >> 1) + 8 * h_r + 4 * (a_r & 1) + b_r;
-    const int first_row = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+    const int first_row = nva_first_key(pos, window, key_chunk);
     const float c_exp = scale * 1.4426950408889634f;      // scale * log2(e)
 
     // ---- the request's block table entries for the keys this workgroup reads, once, into LDS
@@ -215,7 +217,8 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     // in scalar registers, plus an offset per lane that never changes.
     const int last_key = kb_hi - 1;
     // whole tiles: kb in [a_end, b_end)
-    const int whole_lo = window > 0 ? (first_any + PF_BM + PF_BN - 1) & ~(PF_BN - 1) : kb_lo;
+    // (from the first key of the tile's last row on, every row sees a tile whole: the first key never decreases)
+    const int whole_lo = window > 0 || key_chunk > 0 ? (nva_first_key(last_pos, window, key_chunk) + PF_BN - 1) & ~(PF_BN - 1) : kb_lo;
     const int whole_hi = (start + q0 + 1) & ~(PF_BN - 1);
     const int a_end = min(max(whole_lo, kb_lo), (kb_hi + PF_BN - 1) & ~(PF_BN - 1));
     const int b_end = max(a_end, min(whole_hi, kb_hi));
@@ -539,7 +542,7 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
                                      const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                      int table_stride, const int32_t* cu_seqlens_q, const int32_t* kv_lens,
                                      const int32_t* tiles, int64_t num_tiles, int num_q_heads,
-                                     int num_kv_heads, int head_dim, int page_size, float scale, int window,
+                                     int num_kv_heads, int head_dim, int page_size, float scale, int window, int chunk,
                                      const float* sinks, int32_t* error_flag, hipStream_t stream) {
     if (num_tiles == 0) return 0;
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
@@ -556,7 +559,7 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
     }
     const int G = num_q_heads / num_kv_heads;
     const int64_t grid_y = (int64_t)num_kv_heads * ((G + PF_WAVES - 1) / PF_WAVES);
-    if (!tiles || num_tiles < 0 || num_tiles * grid_y > 0x7fffffff || window < 0 || table_stride <= 0)
+    if (!tiles || num_tiles < 0 || num_tiles * grid_y > 0x7fffffff || window < 0 || chunk < 0 || table_stride <= 0)
         return nva_fail("attn_prefill: bad sizes (tiles %lld, heads %lld)", (long long)num_tiles, (long long)grid_y);
     if (table_stride > 4096) {
         nva_fail("attn_prefill: block tables of %d pages do not fit the kernel's staging buffer", table_stride);
@@ -580,7 +583,7 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
                        (const __bf16*)q, q_stride, (__bf16*)out, out_stride, (const __bf16*)k_cache,                 \
                        (const __bf16*)v_cache, block_tables, table_stride, cu_seqlens_q, kv_lens, tiles,             \
                        (int)num_tiles, SS == 1 && PF_WAVES_PER_SIMD(DD) == 2 && total <= 2 * cus ? (int)total : 0,   \
-                       num_q_heads, num_kv_heads, page_size, scale, window, sinks, error_flag)
+                       num_q_heads, num_kv_heads, page_size, scale, window, chunk, sinks, error_flag)
 #define LAUNCH(DD)                                                                                                 \
     do {                                                                                                           \
         if (PF_WAVES_PER_SIMD(DD) == 2 && two_sets) LAUNCH_SETS(DD, PF_WAVES_PER_SIMD(DD));                         \

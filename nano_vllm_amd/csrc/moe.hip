@@ -24,6 +24,18 @@
 #define MOE_BK 32
 #define MOE_MAX_EXPERTS 1024
 
+// The largest value among the lanes' candidates and its index (of equal values the lower index), in all lanes.
+__device__ __forceinline__ void moe_wave_best(float& v, int& idx) {
+#pragma unroll
+    for (int off = NVA_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(v, off, NVA_WAVE);
+        const int oi = __shfl_xor(idx, off, NVA_WAVE);
+        if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+    }
+}
+
+// One wave per token: a lane looks after the experts (and groups) lane, lane + 64, ...; every choice is a
+// maximum over the wave.
 __global__ void __launch_bounds__(NVA_WAVE)
 moe_route_kernel(const float* __restrict__ logits, int64_t stride, int experts, int top, int group_count, int group_keep,
                  float scale, int32_t* __restrict__ ids, float* __restrict__ weights) {
@@ -32,35 +44,48 @@ moe_route_kernel(const float* __restrict__ logits, int64_t stride, int experts, 
     __shared__ unsigned char open_s[MOE_MAX_EXPERTS];
     const int64_t t = blockIdx.x;
     const int lane = threadIdx.x;
-    for (int e = lane; e < experts; e += NVA_WAVE) s_s[e] = 1.f / (1.f + expf(-logits[t * stride + e]));
+    const bool all_groups = group_keep == group_count;
+    for (int e = lane; e < experts; e += NVA_WAVE) {
+        s_s[e] = 1.f / (1.f + expf(-logits[t * stride + e]));
+        open_s[e] = all_groups ? 1 : 0;
+    }
     __syncthreads();
     const int per = experts / group_count;
-    for (int g = lane; g < group_count; g += NVA_WAVE) {
-        float a = -INFINITY, b = -INFINITY;          // the two largest of the group
-        for (int i = 0; i < per; ++i) {
-            const float v = s_s[g * per + i];
-            if (v > a) { b = a; a = v; } else if (v > b) b = v;
+    if (!all_groups) {
+        for (int g = lane; g < group_count; g += NVA_WAVE) {
+            float a = -INFINITY, b = -INFINITY;      // the two largest of the group
+            for (int i = 0; i < per; ++i) {
+                const float v = s_s[g * per + i];
+                if (v > a) { b = a; a = v; } else if (v > b) b = v;
+            }
+            g_s[g] = per > 1 ? a + b : a;
         }
-        g_s[g] = per > 1 ? a + b : a;
-    }
-    for (int e = lane; e < experts; e += NVA_WAVE) open_s[e] = 0;
-    __syncthreads();
-    if (lane == 0) {
+        __syncthreads();
         for (int k = 0; k < group_keep; ++k) {
-            int best = 0;
-            for (int g = 1; g < group_count; ++g)
-                if (g_s[g] > g_s[best]) best = g;
-            g_s[best] = -INFINITY;
-            for (int i = 0; i < per; ++i) open_s[best * per + i] = 1;
+            float v = -INFINITY;
+            int best = 0x7fffffff;
+            for (int g = lane; g < group_count; g += NVA_WAVE)
+                if (g_s[g] > v) { v = g_s[g]; best = g; }
+            moe_wave_best(v, best);
+            __syncthreads();
+            if (lane == 0) g_s[best] = -INFINITY;
+            for (int i = lane; i < per; i += NVA_WAVE) open_s[best * per + i] = 1;
+            __syncthreads();
         }
-        for (int k = 0; k < top; ++k) {
-            int best = -1;
-            for (int e = 0; e < experts; ++e)
-                if (open_s[e] && (best < 0 || s_s[e] > s_s[best])) best = e;
+    }
+    for (int k = 0; k < top; ++k) {
+        float v = -INFINITY;
+        int best = 0x7fffffff;
+        for (int e = lane; e < experts; e += NVA_WAVE)
+            if (open_s[e] && s_s[e] > v) { v = s_s[e]; best = e; }
+        moe_wave_best(v, best);
+        __syncthreads();
+        if (lane == 0) {
             open_s[best] = 0;
             ids[t * top + k] = best;
-            weights[t * top + k] = scale * s_s[best];
+            weights[t * top + k] = scale * v;
         }
+        __syncthreads();
     }
 }
 
@@ -68,7 +93,7 @@ moe_route_kernel(const float* __restrict__ logits, int64_t stride, int experts, 
 // of its expert depends on the order in which the threads arrive; no result does, since every row of the
 // products is computed by itself.
 __global__ void __launch_bounds__(1024)
-moe_plan_kernel(const int32_t* __restrict__ ids, int64_t pairs, int experts, int32_t* __restrict__ place,
+moe_plan_kernel(const int32_t* __restrict__ ids, int64_t pairs, int experts, int bm, int32_t* __restrict__ place,
                 int32_t* __restrict__ rows, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
                 int32_t* __restrict__ tile_rows, int32_t* __restrict__ num_tiles) {
     __shared__ int count_s[MOE_MAX_EXPERTS], cursor_s[MOE_MAX_EXPERTS], begin_s[MOE_MAX_EXPERTS], tile0_s[MOE_MAX_EXPERTS];
@@ -82,17 +107,17 @@ moe_plan_kernel(const int32_t* __restrict__ ids, int64_t pairs, int experts, int
             begin_s[e] = at;
             tile0_s[e] = tiles;
             at += count_s[e];
-            tiles += (count_s[e] + MOE_BM - 1) / MOE_BM;
+            tiles += (count_s[e] + bm - 1) / bm;
         }
         num_tiles[0] = tiles;
     }
     __syncthreads();
     for (int e = threadIdx.x; e < experts; e += blockDim.x) {
         const int n = count_s[e];
-        for (int i = 0; i * MOE_BM < n; ++i) {
+        for (int i = 0; i * bm < n; ++i) {
             tile_expert[tile0_s[e] + i] = e;
-            tile_row0[tile0_s[e] + i] = begin_s[e] + i * MOE_BM;
-            tile_rows[tile0_s[e] + i] = min(MOE_BM, n - i * MOE_BM);
+            tile_row0[tile0_s[e] + i] = begin_s[e] + i * bm;
+            tile_rows[tile0_s[e] + i] = min(bm, n - i * bm);
         }
     }
     for (int64_t i = threadIdx.x; i < pairs; i += blockDim.x) {
@@ -158,6 +183,87 @@ moe_tile_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__
     }
 }
 
+#if defined(NVA_BF16)
+// ---------------------------------------------------------------------------- the tile product on the matrix cores
+// A workgroup of four waves takes a tile of BM rows (of one expert) and 4 * WR outputs: a wave 16 or 32 rows of the
+// expert's matrix as the A operand of v_mfma_f32_16x16x32_bf16, straight from global memory into registers (a lane 16
+// bytes of a row a load; every byte of the matrix is read once per tile of rows), and all BM rows of x as B operands
+// from LDS, where the tile's rows are gathered a chunk of MOE_KC columns at a time.  A row's sum over k runs in the
+// order of the chunks whatever the tile it fell into.
+typedef __attribute__((ext_vector_type(8))) __bf16 moe_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float moe_f32x4;
+#define MOE_KC 128
+
+template <int BM, int WR, bool UP>
+__global__ void __launch_bounds__(256)
+moe_mfma_kernel(const __bf16* __restrict__ a, int64_t a_stride, const __bf16* __restrict__ w, int n, int k,
+                const int32_t* __restrict__ rows, int top, const int32_t* __restrict__ tile_expert,
+                const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ tile_rows,
+                const int32_t* __restrict__ num_tiles, int act, __bf16* __restrict__ out, int64_t out_stride) {
+    constexpr int MB = BM / 16, FR = WR / 16, XS = MOE_KC + 8;
+    __shared__ __attribute__((aligned(16))) __bf16 x_s[BM * XS];
+    __shared__ int src_s[BM];
+    const int tile = blockIdx.x;
+    if (tile >= num_tiles[0]) return;
+    const int e = tile_expert[tile], row0 = tile_row0[tile], nrows = tile_rows[tile];
+    const int tid = threadIdx.x, wave = tid / NVA_WAVE, lane = tid % NVA_WAVE, col = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.y * 4 * WR + wave * WR;
+    if (tid < BM) src_s[tid] = tid < nrows ? (UP ? rows[row0 + tid] / top : row0 + tid) : -1;
+    const __bf16* we = w + (int64_t)e * n * k;
+    const __bf16* wrow[FR];
+#pragma unroll
+    for (int f = 0; f < FR; ++f) wrow[f] = we + (int64_t)min(n0 + 16 * f + col, n - 1) * k + 8 * g;
+    moe_f32x4 acc[FR][MB];
+#pragma unroll
+    for (int f = 0; f < FR; ++f)
+#pragma unroll
+        for (int b = 0; b < MB; ++b) acc[f][b] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+    const int k_last = k - 8;                      // k is a multiple of 8 (checked by the launcher)
+    for (int k0 = 0; k0 < k; k0 += MOE_KC) {
+        // the chunk's part of the matrix is asked for first, then x is gathered
+        moe_bf16x8 fa[MOE_KC / 32][FR];
+#pragma unroll
+        for (int c = 0; c < MOE_KC / 32; ++c)
+#pragma unroll
+            for (int f = 0; f < FR; ++f) fa[c][f] = *reinterpret_cast<const moe_bf16x8*>(wrow[f] + min(k0 + 32 * c, k_last - 8 * g));
+        __syncthreads();                           // the chunk before is done with (and src_s is written)
+        for (int idx = tid; idx < BM * (MOE_KC / 8); idx += 256) {
+            const int r = idx / (MOE_KC / 8), piece = idx % (MOE_KC / 8);
+            const int kk = k0 + piece * 8;
+            moe_bf16x8 v;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = (__bf16)0.f;
+            if (src_s[r] >= 0 && kk < k) v = *reinterpret_cast<const moe_bf16x8*>(a + (int64_t)src_s[r] * a_stride + kk);
+            *reinterpret_cast<moe_bf16x8*>(&x_s[r * XS + piece * 8]) = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < MOE_KC / 32; ++c) {
+            if (k0 + 32 * c >= k) break;           // (columns of x beyond k are zero, the matrix's clamped)
+#pragma unroll
+            for (int b = 0; b < MB; ++b) {
+                const moe_bf16x8 fb = *reinterpret_cast<const moe_bf16x8*>(&x_s[(16 * b + col) * XS + 32 * c + 8 * g]);
+#pragma unroll
+                for (int f = 0; f < FR; ++f) acc[f][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[c][f], fb, acc[f][b], 0, 0, 0);
+            }
+        }
+    }
+    // acc[f][b][i] = out[row 16 b + col][n0 + 16 f + 4 g + i]
+#pragma unroll
+    for (int f = 0; f < FR; ++f)
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            const int r = 16 * b + col;
+            if (r >= nrows) continue;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int c = n0 + 16 * f + 4 * g + i;
+                if (c < n) out[(int64_t)(row0 + r) * out_stride + c] = (__bf16)(UP ? nva_gate_act(act, acc[f][b][i]) : acc[f][b][i]);
+            }
+        }
+}
+#endif
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(const T* __restrict__ o, int64_t o_stride, const int32_t* __restrict__ place,
@@ -187,8 +293,15 @@ NVA_EXPORT int NVA_NAME(nva_moe_route)(const float* logits, int64_t stride, int6
     return nva_check_launch("moe_route");
 }
 
-// Rows of a tile of the experts' products (the plan's arrays are sized with it).
-NVA_EXPORT int NVA_NAME(nva_moe_tile_rows)() { return MOE_BM; }
+// Rows of a tile of the experts' products for this many pairs (token, choice) and experts: the plan's arrays are
+// sized with it.  Many rows an expert: tall tiles, so that an expert's matrix is read few times.
+static int moe_tile_rows(int64_t pairs, int experts, int k, int ff) {
+#if defined(NVA_BF16)
+    if (k % 8 == 0 && ff % 8 == 0) return pairs >= 64 * (int64_t)experts ? 128 : 32;
+#endif
+    return MOE_BM;
+}
+NVA_EXPORT int NVA_NAME(nva_moe_tile_rows)(int64_t pairs, int experts, int k, int ff) { return moe_tile_rows(pairs, experts, k, ff); }
 
 // x [tokens, k] elements; ids, weights [tokens, top]; up [E * ff, k], down [E * k, ff] elements; add [tokens, k] or null.
 // Scratch: place, rows int32 [tokens * top]; tiles int32 [3 * max_tiles + 1] with max_tiles = tokens * top / MOE_BM + E
@@ -202,8 +315,9 @@ NVA_EXPORT int NVA_NAME(nva_moe_experts)(const void* x, int64_t x_stride, const 
     const int64_t pairs = tokens * top;
     if (tokens < 0 || top <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || k <= 0 || ff <= 0 || pairs > 0x7fffffff)
         return nva_fail("moe_experts: bad sizes tokens=%lld top=%d experts=%d k=%d ff=%d", (long long)tokens, top, experts, k, ff);
-    if (max_tiles < pairs / MOE_BM + experts || max_tiles > 0x7fffffff)
-        return nva_fail("moe_experts: room for %lld tiles, %lld may be needed", (long long)max_tiles, (long long)(pairs / MOE_BM + experts));
+    const int bm = moe_tile_rows(pairs, experts, k, ff);
+    if (max_tiles < pairs / bm + experts || max_tiles > 0x7fffffff)
+        return nva_fail("moe_experts: room for %lld tiles, %lld may be needed", (long long)max_tiles, (long long)(pairs / bm + experts));
     if (act < 0 || act > 3) return nva_fail("moe_experts: unknown activation %d", act);
     if (!x || !ids || !weights || !up || !down || !place || !rows || !tiles || !hidden || !outs || !y)
         return nva_fail("moe_experts: a tensor is missing");
@@ -211,15 +325,31 @@ NVA_EXPORT int NVA_NAME(nva_moe_experts)(const void* x, int64_t x_stride, const 
     int32_t* tile_row0 = tiles + max_tiles;
     int32_t* tile_rows = tiles + 2 * max_tiles;
     int32_t* num_tiles = tiles + 3 * max_tiles;
-    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, place, rows, tile_expert,
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, stream, ids, pairs, experts, bm, place, rows, tile_expert,
                        tile_row0, tile_rows, num_tiles);
     if ((ff + MOE_BN - 1) / MOE_BN > 65535 || (k + MOE_BN - 1) / MOE_BN > 65535) return nva_fail("moe_experts: too wide");
+#if defined(NVA_BF16)
+    if (k % 8 == 0 && ff % 8 == 0 && x_stride % 8 == 0 && nva_aligned(x, 16) && nva_aligned(up, 16) && nva_aligned(down, 16) &&
+        nva_aligned(hidden, 16)) {
+#define MOE_LAUNCH(BMV, WRV)                                                                                                  \
+        hipLaunchKernelGGL((moe_mfma_kernel<BMV, WRV, true>), dim3((unsigned)max_tiles, (ff + 4 * WRV - 1) / (4 * WRV)),        \
+                           dim3(256), 0, stream, (const __bf16*)x, x_stride, (const __bf16*)up, ff, k, rows, top, tile_expert, \
+                           tile_row0, tile_rows, num_tiles, act, (__bf16*)hidden, (int64_t)ff);                                 \
+        hipLaunchKernelGGL((moe_mfma_kernel<BMV, WRV, false>), dim3((unsigned)max_tiles, (k + 4 * WRV - 1) / (4 * WRV)),        \
+                           dim3(256), 0, stream, (const __bf16*)hidden, (int64_t)ff, (const __bf16*)down, k, ff, rows, top,     \
+                           tile_expert, tile_row0, tile_rows, num_tiles, act, (__bf16*)outs, (int64_t)k)
+        if (bm == 128) { MOE_LAUNCH(128, 32); } else { MOE_LAUNCH(32, 16); }
+#undef MOE_LAUNCH
+    } else
+#endif
+    {
     hipLaunchKernelGGL((moe_tile_kernel<elem_t, true>), dim3((unsigned)max_tiles, (ff + MOE_BN - 1) / MOE_BN), dim3(256), 0,
                        stream, (const elem_t*)x, x_stride, (const elem_t*)up, ff, k, rows, top, tile_expert, tile_row0,
                        tile_rows, num_tiles, act, (elem_t*)hidden, (int64_t)ff);
     hipLaunchKernelGGL((moe_tile_kernel<elem_t, false>), dim3((unsigned)max_tiles, (k + MOE_BN - 1) / MOE_BN), dim3(256), 0,
                        stream, (const elem_t*)hidden, (int64_t)ff, (const elem_t*)down, k, ff, rows, top, tile_expert,
                        tile_row0, tile_rows, num_tiles, act, (elem_t*)outs, (int64_t)k);
+    }
     for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
         const unsigned nt = (unsigned)((tokens - t0) < 65535 ? (tokens - t0) : 65535);
         hipLaunchKernelGGL((moe_combine_kernel<elem_t>), dim3((k + 255) / 256, nt), dim3(256), 0, stream, (const elem_t*)outs,

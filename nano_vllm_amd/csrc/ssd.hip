@@ -17,14 +17,15 @@
 //
 // Kernels: conv (a thread per token and channel; a request that brings one token also shifts its kept
 // inputs), conv_state (the kept inputs of requests that bring a portion), scan, finish.  The scan gives
-// every thread one column of S (all N rows, in registers), so the read-out needs no exchange between
-// threads; B and C of a token are staged in LDS for the wave.  A long portion is cut into blocks that
+// every thread one column of S (up to 64 of its rows, in registers: a state of more rows is shared out over
+// 2 or 4 lanes, whose sums meet by shuffles); B, C and x of 16 tokens at a time are staged in LDS for the wave.  A long portion is cut into blocks that
 // run side by side, each from a zero state (the first from the request's); a pass over the blocks makes
 // every block's true state at its end, E_b = exp(sum of the block's log-decays) E_(b-1) + U_b, and a
 // second pass adds what the state before a block contributes, exp(log-decay up to t) E_(b-1)^T C_t.
 #include "common.h"
 
 #define SSD_MAX_TAPS 16
+#define SSD_TB 16          // tokens whose inputs the recurrence stages at a time
 
 __device__ __forceinline__ float ssd_silu(float x) { return x / (1.f + expf(-x)); }
 __device__ __forceinline__ float ssd_softplus(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
@@ -111,7 +112,7 @@ ssd_conv_state_kernel(const T* __restrict__ proj, int64_t stride, int col0, int 
 //         start, in cum[t, h]; the request's state is not written.
 // mode 2 (blocks, second pass): the blocks after a portion's first add exp(cum_t) E^T C_t to y, E the true
 //         state before the block (block_states[u - 1] after the pass over the blocks).
-template <typename T, int NMAX>
+template <typename T, int NPER, int NSPLIT>
 __global__ void __launch_bounds__(NVA_WAVE)
 ssd_scan_kernel(const T* __restrict__ proj, int64_t stride, int dt_col, const T* __restrict__ conv, int channels,
                 int heads, int vdim, int n_state, int groups, const float* __restrict__ dt_bias,
@@ -119,9 +120,15 @@ ssd_scan_kernel(const T* __restrict__ proj, int64_t stride, int dt_col, const T*
                 const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_starts,
                 const int32_t* __restrict__ state_slots, int first_seq, const int32_t* __restrict__ units, int mode,
                 float* __restrict__ block_states, float* __restrict__ cum, float* __restrict__ y) {
-    __shared__ float b_s[NMAX], c_s[NMAX];
+    // B, C, x, the step size and the decay of SSD_TB tokens at a time: their loads are on their way
+    // together, and the tokens of a batch run from LDS
+    __shared__ __attribute__((aligned(16))) float b_s[SSD_TB][NPER * NSPLIT], c_s[SSD_TB][NPER * NSPLIT];
+    __shared__ float x_s[SSD_TB][NVA_WAVE], dt_s[SSD_TB], decay_s[SSD_TB];
+    // a wave's lanes: NSPLIT parts of the state's rows (NPER rows each) times 64 / NSPLIT columns
+    constexpr int NMAX = NPER * NSPLIT, PL = NVA_WAVE / NSPLIT;
     const int u = blockIdx.z, h = blockIdx.y;
-    const int p = blockIdx.x * NVA_WAVE + threadIdx.x;
+    const int part = threadIdx.x / PL, row0 = part * NPER;
+    const int p = blockIdx.x * PL + threadIdx.x % PL;
     const bool mine = p < vdim;
     int s, t0, n, first_block = 1;
     if (units) {
@@ -142,58 +149,82 @@ ssd_scan_kernel(const T* __restrict__ proj, int64_t stride, int dt_col, const T*
     float* own = state + (((int64_t)state_slots[s] * heads + h) * n_state) * vdim + p;
     float* block = block_states ? block_states + (((int64_t)u * heads + h) * n_state) * vdim + p : nullptr;
 
-    float S[NMAX];
+    float S[NPER];                                  // rows row0 .. row0 + NPER - 1 of column p
     if (mode == 2) {
         const float* before = block - (int64_t)heads * n_state * vdim;       // the unit before: the block before
 #pragma unroll
-        for (int i = 0; i < NMAX; ++i) S[i] = mine && i < n_state ? before[(int64_t)i * vdim] : 0.f;
+        for (int i = 0; i < NPER; ++i) S[i] = mine && row0 + i < n_state ? before[(int64_t)(row0 + i) * vdim] : 0.f;
     } else {
         const bool carried = first_block && seq_starts[s] > 0;
 #pragma unroll
-        for (int i = 0; i < NMAX; ++i) S[i] = carried && mine && i < n_state ? own[(int64_t)i * vdim] : 0.f;
+        for (int i = 0; i < NPER; ++i) S[i] = carried && mine && row0 + i < n_state ? own[(int64_t)(row0 + i) * vdim] : 0.f;
     }
+    // the read-out of a column: the sum over the lanes that hold its parts, in all of them
+    auto whole = [&](float v) -> float {
+#pragma unroll
+        for (int off = PL; off < NVA_WAVE; off <<= 1) v += __shfl_xor(v, off, NVA_WAVE);
+        return v;
+    };
     const float rate = -expf(a_log[h]), bias = dt_bias[h], skip = d_skip[h];
     float log_decay = 0.f;
-    for (int i = 0; i < n; ++i) {
-        const int64_t t = t0 + i;
+    const int lane = threadIdx.x;
+    // rows of S beyond the state's are zero and stay so: B and C are zero there, written once
+    for (int idx = lane; idx < SSD_TB * NMAX; idx += NVA_WAVE)
+        if (idx % NMAX >= n_state) b_s[idx / NMAX][idx % NMAX] = c_s[idx / NMAX][idx % NMAX] = 0.f;
+    for (int i0 = 0; i0 < n; i0 += SSD_TB) {
+        const int nb = min(SSD_TB, n - i0);
+        const int64_t tb = t0 + i0;
         __syncthreads();
-        for (int k = threadIdx.x; k < n_state; k += NVA_WAVE) {
-            b_s[k] = to_float(b_col[t * channels + k]);
-            c_s[k] = to_float(c_col[t * channels + k]);
+        for (int idx = lane; idx < nb * n_state; idx += NVA_WAVE) {
+            const int j = idx / n_state, k = idx % n_state;
+            c_s[j][k] = to_float(c_col[(tb + j) * channels + k]);
+            if (mode != 2) b_s[j][k] = to_float(b_col[(tb + j) * channels + k]);
         }
-        __syncthreads();
-        if (mode == 2) {
-            float acc = 0.f;
-#pragma unroll
-            for (int k = 0; k < NMAX; ++k)
-                if (k < n_state) acc += S[k] * c_s[k];
-            if (mine) y[t * inner + h * vdim + p] += expf(cum[t * heads + h]) * acc;
-            continue;
-        }
-        const float dt = ssd_softplus(to_float(proj[t * stride + dt_col + h]) + bias);
-        const float decay = expf(rate * dt);
-        const float x = mine ? to_float(conv[t * channels + h * vdim + p]) : 0.f;
-        const float dx = dt * x;
-        float acc = 0.f;
-#pragma unroll
-        for (int k = 0; k < NMAX; ++k) {
-            if (k < n_state) {
-                S[k] = decay * S[k] + b_s[k] * dx;
-                acc += S[k] * c_s[k];
+        if (mode != 2)
+            for (int j = 0; j < nb; ++j) x_s[j][lane] = mine ? to_float(conv[(tb + j) * channels + h * vdim + p]) : 0.f;   // (a column's lanes hold the same)
+        if (lane < nb) {
+            if (mode == 2) {
+                decay_s[lane] = expf(cum[(tb + lane) * heads + h]);
+            } else {
+                const float dt = ssd_softplus(to_float(proj[(tb + lane) * stride + dt_col + h]) + bias);
+                dt_s[lane] = dt;
+                decay_s[lane] = expf(rate * dt);
             }
         }
-        if (mine) y[t * inner + h * vdim + p] = acc + skip * x;
-        if (mode == 1) {
-            log_decay += rate * dt;
-            if (threadIdx.x == 0 && blockIdx.x == 0) cum[t * heads + h] = log_decay;
+        __syncthreads();
+        for (int j = 0; j < nb; ++j) {
+            const int64_t t = tb + j;
+            if (mode == 2) {
+                float acc = 0.f;
+#pragma unroll
+                for (int k = 0; k < NPER; ++k) acc += S[k] * c_s[j][row0 + k];
+                acc = whole(acc);
+                if (mine && part == 0) y[t * inner + h * vdim + p] += decay_s[j] * acc;
+                continue;
+            }
+            const float dt = dt_s[j], decay = decay_s[j];
+            const float x = x_s[j][lane];
+            const float dx = dt * x;
+            float acc = 0.f;
+#pragma unroll
+            for (int k = 0; k < NPER; ++k) {
+                S[k] = decay * S[k] + b_s[j][row0 + k] * dx;
+                acc += S[k] * c_s[j][row0 + k];
+            }
+            acc = whole(acc);
+            if (mine && part == 0) y[t * inner + h * vdim + p] = acc + skip * x;
+            if (mode == 1) {
+                log_decay += rate * dt;
+                if (lane == 0 && blockIdx.x == 0) cum[t * heads + h] = log_decay;
+            }
         }
     }
     if (mode == 2 || !mine) return;
     // (a portion of one block has no pass over its blocks: its end state is the request's new state)
     float* dst = mode == 1 && units[4 * u + 3] > 1 ? block : own;
 #pragma unroll
-    for (int i = 0; i < NMAX; ++i)
-        if (i < n_state) dst[(int64_t)i * vdim] = S[i];
+    for (int i = 0; i < NPER; ++i)
+        if (row0 + i < n_state) dst[(int64_t)(row0 + i) * vdim] = S[i];
 }
 
 // The pass over a portion's blocks: block_states[b] <- exp(total log-decay of block b) * block_states[b - 1]
@@ -244,14 +275,19 @@ ssd_finish_kernel(const float* __restrict__ y, const T* __restrict__ proj, int64
     }
 }
 
-template <int NMAX>
-static void launch_scan(dim3 grid, hipStream_t stream, const elem_t* proj, int64_t stride, int dt_col, const elem_t* conv,
-                        int channels, int heads, int vdim, int n_state, int groups, const float* dt_bias, const float* a_log,
-                        const float* d_skip, float* state, const int32_t* cu, const int32_t* starts, const int32_t* slots,
-                        int first_seq, const int32_t* units, int mode, float* block_states, float* cum, float* y) {
-    hipLaunchKernelGGL((ssd_scan_kernel<elem_t, NMAX>), grid, dim3(NVA_WAVE), 0, stream, proj, stride, dt_col, conv, channels,
-                       heads, vdim, n_state, groups, dt_bias, a_log, d_skip, state, cu, starts, slots, first_seq, units, mode,
-                       block_states, cum, y);
+struct ScanArgs {
+    const elem_t* proj; int64_t stride; int dt_col; const elem_t* conv; int channels, heads, vdim, n_state, groups;
+    const float *dt_bias, *a_log, *d_skip; float* state; const int32_t *cu, *starts, *slots;
+    float *block_states, *cum, *y;
+};
+
+template <int NPER, int NSPLIT>
+static void launch_scan(const ScanArgs& a, unsigned units, int first_seq, const int32_t* us, int mode, hipStream_t stream) {
+    constexpr int PL = NVA_WAVE / NSPLIT;
+    const dim3 grid((unsigned)((a.vdim + PL - 1) / PL), (unsigned)a.heads, units);
+    hipLaunchKernelGGL((ssd_scan_kernel<elem_t, NPER, NSPLIT>), grid, dim3(NVA_WAVE), 0, stream, a.proj, a.stride, a.dt_col,
+                       a.conv, a.channels, a.heads, a.vdim, a.n_state, a.groups, a.dt_bias, a.a_log, a.d_skip, a.state, a.cu,
+                       a.starts, a.slots, first_seq, us, mode, a.block_states, a.cum, a.y);
 }
 
 // proj: [tokens, 2 H P + 2 G N + H] with rows `stride` apart.  conv_out [tokens, C] (elements), y_raw [tokens, H P]
@@ -294,39 +330,26 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
                            dim3(256), 0, stream, pj, stride, inner, channels, taps, conv_state, cu_seqlens, seq_starts,
                            state_slots, (int)num_single);
     const int dt_col = inner + channels;
-    auto scan = [&](dim3 grid, int first_seq, const int32_t* us, int mode) {
-        if (n_state <= 16)
-            launch_scan<16>(grid, stream, pj, stride, dt_col, (const elem_t*)conv_out, channels, heads, vdim, n_state, groups,
-                            dt_bias, a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, first_seq, us, mode,
-                            block_states, cum, y_raw);
-        else if (n_state <= 32)
-            launch_scan<32>(grid, stream, pj, stride, dt_col, (const elem_t*)conv_out, channels, heads, vdim, n_state, groups,
-                            dt_bias, a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, first_seq, us, mode,
-                            block_states, cum, y_raw);
-        else if (n_state <= 64)
-            launch_scan<64>(grid, stream, pj, stride, dt_col, (const elem_t*)conv_out, channels, heads, vdim, n_state, groups,
-                            dt_bias, a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, first_seq, us, mode,
-                            block_states, cum, y_raw);
-        else if (n_state <= 128)
-            launch_scan<128>(grid, stream, pj, stride, dt_col, (const elem_t*)conv_out, channels, heads, vdim, n_state, groups,
-                             dt_bias, a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, first_seq, us, mode,
-                             block_states, cum, y_raw);
-        else
-            launch_scan<256>(grid, stream, pj, stride, dt_col, (const elem_t*)conv_out, channels, heads, vdim, n_state, groups,
-                             dt_bias, a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, first_seq, us, mode,
-                             block_states, cum, y_raw);
+    const ScanArgs args{pj, stride, dt_col, (const elem_t*)conv_out, channels, heads, vdim, n_state, groups, dt_bias, a_log,
+                        d_skip, state, cu_seqlens, seq_starts, state_slots, block_states, cum, y_raw};
+    // a thread holds up to 64 rows of a column of S; a state of more rows is shared out over 2 or 4 lanes
+    auto scan = [&](unsigned units, int first_seq, const int32_t* us, int mode) {
+        if (n_state <= 16) launch_scan<16, 1>(args, units, first_seq, us, mode, stream);
+        else if (n_state <= 32) launch_scan<32, 1>(args, units, first_seq, us, mode, stream);
+        else if (n_state <= 64) launch_scan<64, 1>(args, units, first_seq, us, mode, stream);
+        else if (n_state <= 128) launch_scan<64, 2>(args, units, first_seq, us, mode, stream);
+        else launch_scan<64, 4>(args, units, first_seq, us, mode, stream);
     };
-    const unsigned px = (unsigned)((vdim + NVA_WAVE - 1) / NVA_WAVE);
     if (n_chains) {
         if (n_units <= 0 || n_units > 65535) return nva_fail("state_space: bad block count %lld", (long long)n_units);
-        if (num_single) scan(dim3(px, heads, (unsigned)num_single), 0, nullptr, 0);
-        scan(dim3(px, heads, (unsigned)n_units), (int)num_single, units, 1);
+        if (num_single) scan((unsigned)num_single, 0, nullptr, 0);
+        scan((unsigned)n_units, (int)num_single, units, 1);
         hipLaunchKernelGGL(ssd_chain_kernel, dim3((n_state * vdim + 255) / 256, heads, (unsigned)n_chains), dim3(256), 0, stream,
                            block_states, cum, state, chains, units, cu_seqlens, state_slots, (int)num_single, heads, n_state,
                            vdim);
-        scan(dim3(px, heads, (unsigned)n_units), (int)num_single, units, 2);
+        scan((unsigned)n_units, (int)num_single, units, 2);
     } else {
-        scan(dim3(px, heads, (unsigned)seqs), 0, nullptr, 0);
+        scan((unsigned)seqs, 0, nullptr, 0);
     }
     const int group_size = inner / norm_groups;
     hipLaunchKernelGGL((ssd_finish_kernel<elem_t>), dim3((unsigned)tokens, norm_groups), dim3(256), 0, stream, y_raw, pj,

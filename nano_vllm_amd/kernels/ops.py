@@ -571,8 +571,8 @@ class HipKernels:
             if (arows, aw) != (tokens, k) or add.dtype != x.dtype:
                 raise KernelError("moe_experts: the addend does not match the input")
         pairs = tokens * top
-        tile_rows = library.load("moe", self.suffix)
-        bm = int(getattr(tile_rows, f"nva_moe_tile_rows_{self.suffix}")())
+        tile_rows = getattr(library.load("moe", self.suffix), f"nva_moe_tile_rows_{self.suffix}")
+        bm = int(tile_rows(c_i64(pairs), c_i32(num_experts), c_i32(k), c_i32(ff)))
         max_tiles = pairs // bm + num_experts
         ints = torch.empty(2 * pairs + 3 * max_tiles + 1, dtype=torch.int32, device=x.device)
         hidden = torch.empty((pairs, ff), dtype=x.dtype, device=x.device)
@@ -1182,13 +1182,12 @@ class HipKernels:
         # them where its shape limits allow; everything else runs the general kernel
         start = 0
         # (the matrix-core kernels fold the scale into the exponent, which needs it positive)
-        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim \
-            and not chunk
+        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf") and v_dim == head_dim
         if batch.num_decode > 0 and mfma and \
                 self._decode_kernel_takes(num_heads // num_kv_heads, head_dim, page_size, q, qs, out, os_):
             start = batch.num_decode
             self._attention_decode(q, qs, out, os_, k_cache, v_cache, tables, batch, start, num_heads, num_kv_heads,
-                                   head_dim, page_size, scale, window, sinks)
+                                   head_dim, page_size, scale, window, sinks, chunk)
         if start < tokens and mfma and start == batch.num_decode and \
                 self._prefill_kernel_takes(head_dim, page_size, tables.shape[1], q, qs, out, os_):
             # portions of prompts: the matrix-core prefill kernel, one workgroup per 32 query rows
@@ -1197,7 +1196,7 @@ class HipKernels:
                          _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.cu_seqlens_q), _p(batch.kv_lens),
                          _p(tiles), c_i64(tiles.shape[0]), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
-                         _p(sinks), _p(self.fault_flag), self._stream())
+                         c_i32(chunk or 0), _p(sinks), _p(self.fault_flag), self._stream())
             start = tokens
         if self.tiled_general_attention and start <= batch.num_decode < tokens and not window and \
                 max(head_dim, v_dim) <= GENERAL_TILED_MAX_HEAD_DIM:
@@ -1412,7 +1411,7 @@ class HipKernels:
                                                                              out_stride)
 
     def _attention_decode(self, q, qs, out, os_, k_cache, v_cache, tables, batch, n, num_heads, num_kv_heads,
-                          head_dim, page_size, scale, window, sinks=None):
+                          head_dim, page_size, scale, window, sinks=None, chunk=None):
         # The work is shared out on the device from the tokens' positions, once per step and (kv
         # heads, window): the first layer that asks makes the plan, the others find it on the batch.
         # The library says how large the partial results may get for this many tokens of at most
@@ -1422,7 +1421,7 @@ class HipKernels:
             plans = batch.step_cache = {}
         for t0 in range(0, n, 1024):
             t1 = min(n, t0 + 1024)
-            key = ("decode_plan", t0, num_kv_heads, head_dim, page_size, window or 0)
+            key = ("decode_plan", t0, num_kv_heads, head_dim, page_size, window or 0, chunk or 0)
             if key not in plans:
                 bound, waves, ints = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int64(0)
                 library.call("attn_decode", "bf16", "nva_attn_decode_plan_size", c_i32(batch.max_kv_len), c_i64(t1 - t0),
@@ -1431,7 +1430,7 @@ class HipKernels:
                 plan = torch.empty(ints.value, dtype=torch.int32, device=q.device)
                 library.call("attn_decode", "bf16", "nva_attn_decode_plan", _p(batch.positions[t0:t1]),
                              _p(batch.token_seq[t0:t1]), c_i64(t1 - t0),
-                             c_i32(num_kv_heads), c_i32(page_size), c_i32(window or 0), c_i32(bound.value),
+                             c_i32(num_kv_heads), c_i32(page_size), c_i32(window or 0), c_i32(chunk or 0), c_i32(bound.value),
                              c_i32(waves.value), _p(plan), _p(self.fault_flag), self._stream())
                 plans[key] = (plan, bound.value, waves.value)
             plan, bound, waves = plans[key]
@@ -1440,7 +1439,7 @@ class HipKernels:
                          _p(scratch), _p(plan), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
                          c_i64(t1 - t0), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
-                         c_i32(bound), c_i32(waves), _p(sinks), _p(self.fault_flag), self._stream())
+                         c_i32(chunk or 0), c_i32(bound), c_i32(waves), _p(sinks), _p(self.fault_flag), self._stream())
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:

@@ -486,7 +486,8 @@ def test_the_choice_of_experts(backend, experts, top, count, keep):
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("tokens,width,ff,experts,top", [(1, 48, 20, 6, 2), (7, 20, 9, 5, 3), (150, 72, 30, 12, 2), (33, 128, 64, 8, 3)])
+@pytest.mark.parametrize("tokens,width,ff,experts,top", [(1, 48, 20, 6, 2), (7, 20, 9, 5, 3), (150, 72, 30, 12, 2), (33, 128, 64, 8, 3),
+                                                         (40, 72, 40, 6, 2), (300, 64, 32, 4, 2), (700, 160, 104, 5, 2), (8, 256, 128, 32, 6)])
 def test_the_experts_products(backend, dtype, tokens, width, ff, experts, top):
     k, dev = _kernels(backend, dtype)
     g = torch.Generator().manual_seed(tokens)
@@ -495,8 +496,9 @@ def test_the_experts_products(backend, dtype, tokens, width, ff, experts, top):
     down = (torch.randn((experts * width, ff), generator=g) * 0.3).to(dtype)
     ids = torch.stack([torch.randperm(experts, generator=g)[:top] for _ in range(tokens)]).to(torch.int32)
     if tokens > 100:
-        ids[:90, 0] = 3                                  # one expert with more rows than a tile holds
-        ids[:90, 1] = 4
+        ids[:90, 0] = experts - 1                        # two experts with more rows than a tile holds
+        ids[:90, 1] = experts - 2
+        ids[:90, 2:] = torch.arange(top - 2)[None, :]
     weights = torch.rand((tokens, top), generator=g) + 0.2
     add = torch.randn((tokens, width), generator=g).to(dtype)
     w = {}
