@@ -201,7 +201,10 @@ moe_mfma_kernel(const __bf16* __restrict__ a, int64_t a_stride, const __bf16* __
                 const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ tile_rows,
                 const int32_t* __restrict__ num_tiles, int act, __bf16* __restrict__ out, int64_t out_stride) {
     constexpr int MB = BM / 16, FR = WR / 16, XS = MOE_KC + 8;
-    __shared__ __attribute__((aligned(16))) __bf16 x_s[BM * XS];
+    constexpr int KS = MOE_KC / 32;                         // products' steps of 32 columns in a chunk
+    constexpr int XP = BM * (MOE_KC / 8) / 256;             // 16-byte pieces of a chunk of x a thread gathers
+    static_assert(BM * (MOE_KC / 8) % 256 == 0, "the pieces of a chunk of x divide among the threads");
+    __shared__ __attribute__((aligned(16))) __bf16 x_s[2][BM * XS];      // two chunks: one multiplied, one arriving
     __shared__ int src_s[BM];
     const int tile = blockIdx.x;
     if (tile >= num_tiles[0]) return;
@@ -209,44 +212,72 @@ moe_mfma_kernel(const __bf16* __restrict__ a, int64_t a_stride, const __bf16* __
     const int tid = threadIdx.x, wave = tid / NVA_WAVE, lane = tid % NVA_WAVE, col = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.y * 4 * WR + wave * WR;
     if (tid < BM) src_s[tid] = tid < nrows ? (UP ? rows[row0 + tid] / top : row0 + tid) : -1;
+    __syncthreads();
     const __bf16* we = w + (int64_t)e * n * k;
     const __bf16* wrow[FR];
 #pragma unroll
     for (int f = 0; f < FR; ++f) wrow[f] = we + (int64_t)min(n0 + 16 * f + col, n - 1) * k + 8 * g;
+    // the rows of x this thread gathers: piece i is row (tid + 256 i) / (MOE_KC / 8), columns 8 ((tid + 256 i) % (MOE_KC / 8))
+    const __bf16* xsrc[XP];
+    int xcol[XP];
+#pragma unroll
+    for (int i = 0; i < XP; ++i) {
+        const int idx = tid + 256 * i, r = idx / (MOE_KC / 8);
+        xcol[i] = (idx % (MOE_KC / 8)) * 8;
+        xsrc[i] = src_s[r] >= 0 ? a + (int64_t)src_s[r] * a_stride + xcol[i] : nullptr;
+    }
     moe_f32x4 acc[FR][MB];
 #pragma unroll
     for (int f = 0; f < FR; ++f)
 #pragma unroll
         for (int b = 0; b < MB; ++b) acc[f][b] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
     const int k_last = k - 8;                      // k is a multiple of 8 (checked by the launcher)
-    for (int k0 = 0; k0 < k; k0 += MOE_KC) {
-        // the chunk's part of the matrix is asked for first, then x is gathered
-        moe_bf16x8 fa[MOE_KC / 32][FR];
+    // (two sets of registers for the matrix's part, named apart so that neither is ever indexed at run time)
+    moe_bf16x8 fa0[KS][FR], fa1[KS][FR], xr[XP];
+    auto ask = [&](int k0, moe_bf16x8 (&fa)[KS][FR]) __attribute__((always_inline)) {   // a chunk's part of the matrix and of x
 #pragma unroll
-        for (int c = 0; c < MOE_KC / 32; ++c)
+        for (int c = 0; c < KS; ++c)
 #pragma unroll
-            for (int f = 0; f < FR; ++f) fa[c][f] = *reinterpret_cast<const moe_bf16x8*>(wrow[f] + min(k0 + 32 * c, k_last - 8 * g));
-        __syncthreads();                           // the chunk before is done with (and src_s is written)
-        for (int idx = tid; idx < BM * (MOE_KC / 8); idx += 256) {
-            const int r = idx / (MOE_KC / 8), piece = idx % (MOE_KC / 8);
-            const int kk = k0 + piece * 8;
-            moe_bf16x8 v;
+            for (int f = 0; f < FR; ++f)
+                fa[c][f] = *reinterpret_cast<const moe_bf16x8*>(wrow[f] + min(k0 + 32 * c, k_last - 8 * g));
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = (__bf16)0.f;
-            if (src_s[r] >= 0 && kk < k) v = *reinterpret_cast<const moe_bf16x8*>(a + (int64_t)src_s[r] * a_stride + kk);
-            *reinterpret_cast<moe_bf16x8*>(&x_s[r * XS + piece * 8]) = v;
+        for (int i = 0; i < XP; ++i) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) xr[i][q] = (__bf16)0.f;
+            if (xsrc[i] && k0 + xcol[i] < k) xr[i] = *reinterpret_cast<const moe_bf16x8*>(xsrc[i] + k0);
         }
-        __syncthreads();
+    };
+    auto put = [&](__bf16* xs) __attribute__((always_inline)) {           // the gathered chunk of x into LDS
 #pragma unroll
-        for (int c = 0; c < MOE_KC / 32; ++c) {
+        for (int i = 0; i < XP; ++i) {
+            const int idx = tid + 256 * i;
+            *reinterpret_cast<moe_bf16x8*>(&xs[(idx / (MOE_KC / 8)) * XS + xcol[i]]) = xr[i];
+        }
+    };
+    // one chunk: the next one is asked for first and is on its way during this chunk's products
+    auto chunk = [&](int k0, moe_bf16x8 (&fa)[KS][FR], moe_bf16x8 (&fa_next)[KS][FR], const __bf16* xs, __bf16* xs_next)
+                     __attribute__((always_inline)) {
+        const bool more = k0 + MOE_KC < k;
+        if (more) ask(k0 + MOE_KC, fa_next);
+#pragma unroll
+        for (int c = 0; c < KS; ++c) {
             if (k0 + 32 * c >= k) break;           // (columns of x beyond k are zero, the matrix's clamped)
 #pragma unroll
             for (int b = 0; b < MB; ++b) {
-                const moe_bf16x8 fb = *reinterpret_cast<const moe_bf16x8*>(&x_s[(16 * b + col) * XS + 32 * c + 8 * g]);
+                const moe_bf16x8 fb = *reinterpret_cast<const moe_bf16x8*>(&xs[(16 * b + col) * XS + 32 * c + 8 * g]);
 #pragma unroll
                 for (int f = 0; f < FR; ++f) acc[f][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[c][f], fb, acc[f][b], 0, 0, 0);
             }
         }
+        if (more) put(xs_next);                    // (what lay there was read before the last barrier)
+        __syncthreads();
+    };
+    ask(0, fa0);
+    put(x_s[0]);
+    __syncthreads();
+    for (int k0 = 0; k0 < k; k0 += 2 * MOE_KC) {
+        chunk(k0, fa0, fa1, x_s[0], x_s[1]);
+        if (k0 + MOE_KC < k) chunk(k0 + MOE_KC, fa1, fa0, x_s[1], x_s[0]);
     }
     // acc[f][b][i] = out[row 16 b + col][n0 + 16 f + 4 g + i]
 #pragma unroll

@@ -25,6 +25,7 @@
 #include "common.h"
 
 #define SSD_MAX_TAPS 16
+#define SSD_CONV_TOKENS 8 // tokens in a row that a thread of the convolution takes
 #define SSD_TB 16          // tokens whose inputs the recurrence stages at a time
 
 __device__ __forceinline__ float ssd_silu(float x) { return x / (1.f + expf(-x)); }
@@ -37,36 +38,58 @@ ssd_conv_kernel(const T* __restrict__ proj, int64_t stride, int col0, int channe
                 const T* __restrict__ conv_w, const T* __restrict__ conv_b, float* __restrict__ conv_state,
                 const int32_t* __restrict__ token_seq, const int32_t* __restrict__ cu_seqlens,
                 const int32_t* __restrict__ seq_starts, const int32_t* __restrict__ state_slots,
-                T* __restrict__ out) {
-    const int64_t t = blockIdx.x;
+                T* __restrict__ out, float* __restrict__ bc, int np, int n_state, int groups, float* __restrict__ dtd,
+                int heads, int dt_col, const float* __restrict__ dt_bias, const float* __restrict__ a_log, int64_t tokens) {
     const int c = blockIdx.y * blockDim.x + threadIdx.x;
     if (c >= channels) return;
-    const int s = token_seq[t];
-    const int begin = cu_seqlens[s], n = cu_seqlens[s + 1] - begin;
-    const int i = (int)(t - begin);                      // the token's place in its request's portion
-    const bool carried = seq_starts[s] > 0;
+    // a thread takes SSD_CONV_TOKENS tokens in a row with its channel's weights in registers
+    float wt[SSD_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < SSD_MAX_TAPS; ++j)
+        if (j < taps) wt[j] = to_float(conv_w[(int64_t)c * taps + j]);
+    const float bias_c = to_float(conv_b[c]);
     const int hist = taps - 1;
-    float* kept = conv_state + ((int64_t)state_slots[s] * channels + c) * hist;
-    float in[SSD_MAX_TAPS];
+    const int inner = channels - 2 * groups * n_state;
+    for (int64_t t = (int64_t)blockIdx.x * SSD_CONV_TOKENS; t < min(tokens, ((int64_t)blockIdx.x + 1) * SSD_CONV_TOKENS); ++t) {
+        const int s = token_seq[t];
+        const int begin = cu_seqlens[s], n = cu_seqlens[s + 1] - begin;
+        const int i = (int)(t - begin);                      // the token's place in its request's portion
+        const bool carried = seq_starts[s] > 0;
+        float* kept = conv_state + ((int64_t)state_slots[s] * channels + c) * hist;
+        float in[SSD_MAX_TAPS];
 #pragma unroll
-    for (int j = 0; j < SSD_MAX_TAPS; ++j) {
-        if (j >= taps) break;
-        const int src = i - (hist - j);                  // place in the portion of tap j's input
-        if (src >= 0) in[j] = to_float(proj[(t - (hist - j)) * stride + col0 + c]);
-        else in[j] = carried ? kept[i + j] : 0.f;        // hist + src = i + j
-    }
-    float sum = to_float(conv_b[c]);
+        for (int j = 0; j < SSD_MAX_TAPS; ++j) {
+            if (j >= taps) break;
+            const int src = i - (hist - j);                  // place in the portion of tap j's input
+            if (src >= 0) in[j] = to_float(proj[(t - (hist - j)) * stride + col0 + c]);
+            else in[j] = carried ? kept[i + j] : 0.f;        // hist + src = i + j
+        }
+        float sum = bias_c;
 #pragma unroll
-    for (int j = 0; j < SSD_MAX_TAPS; ++j) {
-        if (j >= taps) break;
-        sum += to_float(conv_w[(int64_t)c * taps + j]) * in[j];
-    }
-    out[t * channels + c] = from_float<T>(ssd_silu(sum));
-    if (n == 1) {                                        // a single token: the kept inputs move on by one
+        for (int j = 0; j < SSD_MAX_TAPS; ++j) {
+            if (j >= taps) break;
+            sum += wt[j] * in[j];
+        }
+        const T rounded = from_float<T>(ssd_silu(sum));
+        out[t * channels + c] = rounded;
+        // B and C once more as floats, [token][group][B | C][np] (np rows, those beyond the state's zero): the
+        // recurrence reads them from there.  And, by the first threads, the step size and the decay of
+        // every head: dtd[token][head] = (dt, exp(-exp(A_log) dt)).
+        if (c >= inner) {
+            const int idx = c - inner, gn = groups * n_state;
+            bc[((t * groups + (idx % gn) / n_state) * 2 + idx / gn) * np + idx % n_state] = to_float(rounded);
+        }
+        if (c < heads) {
+            const float dt = ssd_softplus(to_float(proj[t * stride + dt_col + c]) + dt_bias[c]);
+            dtd[(t * heads + c) * 2] = dt;
+            dtd[(t * heads + c) * 2 + 1] = expf(-expf(a_log[c]) * dt);
+        }
+        if (n == 1) {                                        // a single token: the kept inputs move on by one
 #pragma unroll
-        for (int j = 0; j < SSD_MAX_TAPS - 1; ++j) {
-            if (j >= hist) break;
-            kept[j] = in[j + 1];
+            for (int j = 0; j < SSD_MAX_TAPS - 1; ++j) {
+                if (j >= hist) break;
+                kept[j] = in[j + 1];
+            }
         }
     }
 }
@@ -112,18 +135,24 @@ ssd_conv_state_kernel(const T* __restrict__ proj, int64_t stride, int col0, int 
 //         start, in cum[t, h]; the request's state is not written.
 // mode 2 (blocks, second pass): the blocks after a portion's first add exp(cum_t) E^T C_t to y, E the true
 //         state before the block (block_states[u - 1] after the pass over the blocks).
+// B, C, the step size and the decay of a token are the same for all lanes of a wave.  Where a thread holds a whole
+// column of S (NSPLIT 1: up to 128 rows) they are read from global memory by addresses that are the same in
+// every lane, which the compiler turns into scalar loads: they cost no vector register and no LDS, and are
+// operands of the multiply-adds as they are.  Where a column is shared out over lanes, B and C of 16 tokens at a
+// time go through LDS.
 template <typename T, int NPER, int NSPLIT>
 __global__ void __launch_bounds__(NVA_WAVE)
-ssd_scan_kernel(const T* __restrict__ proj, int64_t stride, int dt_col, const T* __restrict__ conv, int channels,
-                int heads, int vdim, int n_state, int groups, const float* __restrict__ dt_bias,
+ssd_scan_kernel(const T* __restrict__ conv, int channels, const float* __restrict__ bc, int np,
+                const float* __restrict__ dtd, int heads, int vdim, int n_state, int groups,
                 const float* __restrict__ a_log, const float* __restrict__ d_skip, float* __restrict__ state,
                 const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_starts,
                 const int32_t* __restrict__ state_slots, int first_seq, const int32_t* __restrict__ units, int mode,
                 float* __restrict__ block_states, float* __restrict__ cum, float* __restrict__ y) {
     // B, C, x, the step size and the decay of SSD_TB tokens at a time: their loads are on their way
     // together, and the tokens of a batch run from LDS
-    __shared__ __attribute__((aligned(16))) float b_s[SSD_TB][NPER * NSPLIT], c_s[SSD_TB][NPER * NSPLIT];
-    __shared__ float x_s[SSD_TB][NVA_WAVE], dt_s[SSD_TB], decay_s[SSD_TB];
+    constexpr bool SC = NSPLIT == 1;
+    __shared__ __attribute__((aligned(16))) float b_s[SC ? 1 : SSD_TB][NPER * NSPLIT], c_s[SC ? 1 : SSD_TB][NPER * NSPLIT];
+    __shared__ float x_s[SSD_TB][NVA_WAVE];
     // a wave's lanes: NSPLIT parts of the state's rows (NPER rows each) times 64 / NSPLIT columns
     constexpr int NMAX = NPER * NSPLIT, PL = NVA_WAVE / NSPLIT;
     const int u = blockIdx.z, h = blockIdx.y;
@@ -142,10 +171,10 @@ ssd_scan_kernel(const T* __restrict__ proj, int64_t stride, int dt_col, const T*
         n = cu_seqlens[s + 1] - t0;
     }
     if (mode == 2 && first_block) return;
-    const int inner = heads * vdim, gn = groups * n_state;
+    const int inner = heads * vdim;
     const int g = h / (heads / groups);
-    const T* b_col = conv + inner + g * n_state;
-    const T* c_col = b_col + gn;
+    const float* bc_g = bc + (int64_t)g * 2 * np;             // token t: + t * groups * 2 * np; C: + np
+    const int64_t bc_stride = (int64_t)groups * 2 * np;
     float* own = state + (((int64_t)state_slots[s] * heads + h) * n_state) * vdim + p;
     float* block = block_states ? block_states + (((int64_t)u * heads + h) * n_state) * vdim + p : nullptr;
 
@@ -165,51 +194,48 @@ ssd_scan_kernel(const T* __restrict__ proj, int64_t stride, int dt_col, const T*
         for (int off = PL; off < NVA_WAVE; off <<= 1) v += __shfl_xor(v, off, NVA_WAVE);
         return v;
     };
-    const float rate = -expf(a_log[h]), bias = dt_bias[h], skip = d_skip[h];
+    const float rate = -expf(a_log[h]), skip = d_skip[h];
     float log_decay = 0.f;
     const int lane = threadIdx.x;
-    // rows of S beyond the state's are zero and stay so: B and C are zero there, written once
-    for (int idx = lane; idx < SSD_TB * NMAX; idx += NVA_WAVE)
-        if (idx % NMAX >= n_state) b_s[idx / NMAX][idx % NMAX] = c_s[idx / NMAX][idx % NMAX] = 0.f;
     for (int i0 = 0; i0 < n; i0 += SSD_TB) {
         const int nb = min(SSD_TB, n - i0);
         const int64_t tb = t0 + i0;
         __syncthreads();
-        for (int idx = lane; idx < nb * n_state; idx += NVA_WAVE) {
-            const int j = idx / n_state, k = idx % n_state;
-            c_s[j][k] = to_float(c_col[(tb + j) * channels + k]);
-            if (mode != 2) b_s[j][k] = to_float(b_col[(tb + j) * channels + k]);
-        }
+        if (!SC)
+            for (int idx = lane; idx < nb * NMAX; idx += NVA_WAVE) {          // (np == NMAX here)
+                const int j = idx / NMAX, k = idx % NMAX;
+                c_s[j][k] = bc_g[(tb + j) * bc_stride + np + k];
+                if (mode != 2) b_s[j][k] = bc_g[(tb + j) * bc_stride + k];
+            }
         if (mode != 2)
             for (int j = 0; j < nb; ++j) x_s[j][lane] = mine ? to_float(conv[(tb + j) * channels + h * vdim + p]) : 0.f;   // (a column's lanes hold the same)
-        if (lane < nb) {
-            if (mode == 2) {
-                decay_s[lane] = expf(cum[(tb + lane) * heads + h]);
-            } else {
-                const float dt = ssd_softplus(to_float(proj[(tb + lane) * stride + dt_col + h]) + bias);
-                dt_s[lane] = dt;
-                decay_s[lane] = expf(rate * dt);
-            }
-        }
         __syncthreads();
-        for (int j = 0; j < nb; ++j) {
+        auto step = [&](int j) __attribute__((always_inline)) {
             const int64_t t = tb + j;
+            // (the constant address space: a load from it at an address that is the same in every lane is a scalar load)
+            typedef const __attribute__((address_space(4))) float* scalar_ptr;
+            scalar_ptr bt_c = (scalar_ptr)(uintptr_t)(bc_g + t * bc_stride), ct_c = bt_c + np;
+            const float* bt_l = &b_s[SC ? 0 : j][row0];
+            const float* ct_l = &c_s[SC ? 0 : j][row0];
+#define SSD_B(k) (SC ? bt_c[k] : bt_l[k])
+#define SSD_C(k) (SC ? ct_c[k] : ct_l[k])
             if (mode == 2) {
                 float acc = 0.f;
 #pragma unroll
-                for (int k = 0; k < NPER; ++k) acc += S[k] * c_s[j][row0 + k];
+                for (int k = 0; k < NPER; ++k) acc += S[k] * SSD_C(k);
                 acc = whole(acc);
-                if (mine && part == 0) y[t * inner + h * vdim + p] += decay_s[j] * acc;
-                continue;
+                if (mine && part == 0) y[t * inner + h * vdim + p] += expf(cum[t * heads + h]) * acc;
+                return;
             }
-            const float dt = dt_s[j], decay = decay_s[j];
+            scalar_ptr dd = (scalar_ptr)(uintptr_t)(dtd + (t * heads + h) * 2);
+            const float dt = dd[0], decay = dd[1];
             const float x = x_s[j][lane];
             const float dx = dt * x;
             float acc = 0.f;
 #pragma unroll
             for (int k = 0; k < NPER; ++k) {
-                S[k] = decay * S[k] + b_s[j][row0 + k] * dx;
-                acc += S[k] * c_s[j][row0 + k];
+                S[k] = decay * S[k] + SSD_B(k) * dx;
+                acc += S[k] * SSD_C(k);
             }
             acc = whole(acc);
             if (mine && part == 0) y[t * inner + h * vdim + p] = acc + skip * x;
@@ -217,8 +243,18 @@ ssd_scan_kernel(const T* __restrict__ proj, int64_t stride, int dt_col, const T*
                 log_decay += rate * dt;
                 if (lane == 0 && blockIdx.x == 0) cum[t * heads + h] = log_decay;
             }
+        };
+        // a full batch with the tokens' numbers known at compile time: the next token's operands can be asked for
+        // during this token's sums
+        if (nb == SSD_TB) {
+#pragma unroll
+            for (int j = 0; j < SSD_TB; ++j) step(j);
+        } else {
+            for (int j = 0; j < nb; ++j) step(j);
         }
     }
+#undef SSD_B
+#undef SSD_C
     if (mode == 2 || !mine) return;
     // (a portion of one block has no pass over its blocks: its end state is the request's new state)
     float* dst = mode == 1 && units[4 * u + 3] > 1 ? block : own;
@@ -254,7 +290,7 @@ ssd_chain_kernel(float* __restrict__ block_states, const float* __restrict__ cum
 
 // ---------------------------------------------------------------------------- gate and grouped norm
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 ssd_finish_kernel(const float* __restrict__ y, const T* __restrict__ proj, int64_t stride, const float* __restrict__ weight,
                   int inner, int group_size, float eps, T* __restrict__ out, int64_t out_stride) {
     __shared__ float scratch[16];
@@ -276,27 +312,38 @@ ssd_finish_kernel(const float* __restrict__ y, const T* __restrict__ proj, int64
 }
 
 struct ScanArgs {
-    const elem_t* proj; int64_t stride; int dt_col; const elem_t* conv; int channels, heads, vdim, n_state, groups;
-    const float *dt_bias, *a_log, *d_skip; float* state; const int32_t *cu, *starts, *slots;
+    const elem_t* conv; int channels; const float* bc; int np; const float* dtd; int heads, vdim, n_state, groups;
+    const float *a_log, *d_skip; float* state; const int32_t *cu, *starts, *slots;
     float *block_states, *cum, *y;
 };
+
+// Rows of B and C per token and group in the float copy the recurrence reads: the rows a thread (or the lanes that
+// share a column) hold, the state's rounded up.
+static int ssd_padded_rows(int n_state) {
+    return n_state <= 16 ? 16 : n_state <= 32 ? 32 : n_state <= 64 ? 64 : n_state <= 128 ? 128 : 256;
+}
+NVA_EXPORT int NVA_NAME(nva_state_space_padded_rows)(int n_state) { return ssd_padded_rows(n_state); }
 
 template <int NPER, int NSPLIT>
 static void launch_scan(const ScanArgs& a, unsigned units, int first_seq, const int32_t* us, int mode, hipStream_t stream) {
     constexpr int PL = NVA_WAVE / NSPLIT;
     const dim3 grid((unsigned)((a.vdim + PL - 1) / PL), (unsigned)a.heads, units);
-    hipLaunchKernelGGL((ssd_scan_kernel<elem_t, NPER, NSPLIT>), grid, dim3(NVA_WAVE), 0, stream, a.proj, a.stride, a.dt_col,
-                       a.conv, a.channels, a.heads, a.vdim, a.n_state, a.groups, a.dt_bias, a.a_log, a.d_skip, a.state, a.cu,
-                       a.starts, a.slots, first_seq, us, mode, a.block_states, a.cum, a.y);
+    hipLaunchKernelGGL((ssd_scan_kernel<elem_t, NPER, NSPLIT>), grid, dim3(NVA_WAVE), 0, stream, a.conv, a.channels, a.bc,
+                       a.np, a.dtd, a.heads, a.vdim, a.n_state, a.groups, a.a_log, a.d_skip, a.state, a.cu, a.starts, a.slots,
+                       first_seq, us, mode, a.block_states, a.cum, a.y);
 }
 
 // proj: [tokens, 2 H P + 2 G N + H] with rows `stride` apart.  conv_out [tokens, C] (elements), y_raw [tokens, H P]
 // and cum [tokens, H] (float) are scratch.  state [slots, H, N, P], conv_state [slots, C, K - 1], float.
 // The first num_single requests bring one token each.  units / chains (with block_states [units, H, N, P]): the
 // portions of the requests from num_single on cut into blocks (units[u] = request counted from num_single, first token,
-// tokens, blocks of the portion; chains[c] = first unit, blocks, request, tokens of the last block, for every
+// tokens, blocks of the portion; shape: 0, or how a state of 65 to 128 rows is held (1: a thread a column, 2: four
+// lanes a column; measurements); chains[c] = first unit, blocks, request, tokens of the last block, for every
 // portion of more than one block); null: every portion runs as one.
-NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void* conv_out, float* y_raw, float* cum, void* out,
+// bc: float [tokens, groups, 2, padded rows] (zero where the padded rows exceed the state's: the caller clears it then),
+// dtd: float [tokens, heads, 2]: scratch as well.
+NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void* conv_out, float* bc, float* dtd,
+                                         float* y_raw, float* cum, void* out,
                                          int64_t out_stride, float* state, float* conv_state, int64_t slots,
                                          const int32_t* token_seq, const int32_t* cu_seqlens, const int32_t* seq_starts,
                                          const int32_t* state_slots, int64_t seqs, int64_t tokens, int64_t num_single,
@@ -304,7 +351,7 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
                                          const void* conv_b, const float* dt_bias, const float* a_log, const float* d_skip,
                                          const float* norm_w, int norm_groups, float eps, const int32_t* units,
                                          int64_t n_units, const int32_t* chains, int64_t n_chains, float* block_states,
-                                         hipStream_t stream) {
+                                         int shape, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || seqs <= 0 || seqs > 65535 || num_single < 0 || num_single > seqs || slots <= 0)
         return nva_fail("state_space: bad counts tokens=%lld requests=%lld", (long long)tokens, (long long)seqs);
@@ -316,27 +363,30 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
     if (n_state > 256) return nva_fail("state_space: a state of %d rows (up to 256 are built)", n_state);
     const int inner = heads * vdim, channels = inner + 2 * groups * n_state;
     if (stride < 2 * inner + 2 * groups * n_state + heads) return nva_fail("state_space: rows too short");
-    if (!proj || !conv_out || !y_raw || !out || !state || (!conv_state && taps > 1) || !token_seq || !cu_seqlens || !seq_starts ||
+    if (!proj || !conv_out || !bc || !dtd || !y_raw || !out || !state || (!conv_state && taps > 1) || !token_seq || !cu_seqlens || !seq_starts ||
         !state_slots || !conv_w || !conv_b || !dt_bias || !a_log || !d_skip || !norm_w)
         return nva_fail("state_space: a tensor is missing");
     if (n_chains && (!units || !chains || !block_states || !cum)) return nva_fail("state_space: blocks need their scratch");
     const elem_t* pj = (const elem_t*)proj;
     if (tokens > 0x7fffffff || (channels + 255) / 256 > 65535) return nva_fail("state_space: too many tokens or channels");
-    hipLaunchKernelGGL((ssd_conv_kernel<elem_t>), dim3((unsigned)tokens, (channels + 255) / 256), dim3(256), 0, stream, pj,
+    hipLaunchKernelGGL((ssd_conv_kernel<elem_t>),
+                       dim3((unsigned)((tokens + SSD_CONV_TOKENS - 1) / SSD_CONV_TOKENS), (channels + 255) / 256), dim3(256), 0, stream, pj,
                        stride, inner, channels, taps, (const elem_t*)conv_w, (const elem_t*)conv_b, conv_state, token_seq,
-                       cu_seqlens, seq_starts, state_slots, (elem_t*)conv_out);
+                       cu_seqlens, seq_starts, state_slots, (elem_t*)conv_out, bc, ssd_padded_rows(n_state), n_state, groups, dtd,
+                       heads, inner + channels, dt_bias, a_log, tokens);
     if (seqs > num_single && taps > 1)
         hipLaunchKernelGGL((ssd_conv_state_kernel<elem_t>), dim3((channels + 255) / 256, (unsigned)(seqs - num_single)),
                            dim3(256), 0, stream, pj, stride, inner, channels, taps, conv_state, cu_seqlens, seq_starts,
                            state_slots, (int)num_single);
-    const int dt_col = inner + channels;
-    const ScanArgs args{pj, stride, dt_col, (const elem_t*)conv_out, channels, heads, vdim, n_state, groups, dt_bias, a_log,
-                        d_skip, state, cu_seqlens, seq_starts, state_slots, block_states, cum, y_raw};
-    // a thread holds up to 64 rows of a column of S; a state of more rows is shared out over 2 or 4 lanes
+    const ScanArgs args{(const elem_t*)conv_out, channels, bc, ssd_padded_rows(n_state), dtd, heads, vdim, n_state, groups,
+                        a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, block_states, cum, y_raw};
+    // a thread holds up to 128 rows of a column of S; a state of more rows is shared out over 4 lanes
     auto scan = [&](unsigned units, int first_seq, const int32_t* us, int mode) {
         if (n_state <= 16) launch_scan<16, 1>(args, units, first_seq, us, mode, stream);
         else if (n_state <= 32) launch_scan<32, 1>(args, units, first_seq, us, mode, stream);
         else if (n_state <= 64) launch_scan<64, 1>(args, units, first_seq, us, mode, stream);
+        else if (n_state <= 128 && shape == 1) launch_scan<128, 1>(args, units, first_seq, us, mode, stream);
+        else if (n_state <= 128 && shape == 2) launch_scan<32, 4>(args, units, first_seq, us, mode, stream);
         else if (n_state <= 128) launch_scan<64, 2>(args, units, first_seq, us, mode, stream);
         else launch_scan<64, 4>(args, units, first_seq, us, mode, stream);
     };
@@ -352,7 +402,9 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
         scan((unsigned)seqs, 0, nullptr, 0);
     }
     const int group_size = inner / norm_groups;
-    hipLaunchKernelGGL((ssd_finish_kernel<elem_t>), dim3((unsigned)tokens, norm_groups), dim3(256), 0, stream, y_raw, pj,
+    // (few tokens: more threads a row, so that a row's loads are on their way at once)
+    hipLaunchKernelGGL((ssd_finish_kernel<elem_t>), dim3((unsigned)tokens, norm_groups),
+                       dim3(tokens <= 64 && group_size >= 2048 ? 1024 : 256), 0, stream, y_raw, pj,
                        stride, norm_w, inner, group_size, eps, (elem_t*)out, out_stride);
     return nva_check_launch("state_space");
 }

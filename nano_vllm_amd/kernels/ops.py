@@ -284,6 +284,9 @@ class HipKernels:
         self.tiled_general_attention = True
         # False: the state-space layer runs a portion's tokens one after the other, whatever its length
         self.state_space_blocks_side_by_side = True
+        # how the recurrence holds a state of 65 to 128 rows: 0 two lanes a column (what serves), 1 a thread a column
+        # with scalar operands, 2 four lanes a column (measurements)
+        self.state_space_shape = 0
 
     # ------------------------------------------------------------------ helpers
     def _stream(self):
@@ -1260,6 +1263,13 @@ class HipKernels:
             raise KernelError("state_space: output does not match")
         conv_out = torch.empty((tokens, channels), dtype=proj.dtype, device=proj.device)
         y_raw = torch.empty((tokens, inner), dtype=torch.float32, device=proj.device)
+        # B and C once more as floats, in rows padded to what a thread of the recurrence holds, and (dt, decay) per head
+        padded = getattr(library.load("ssd", self.suffix), f"nva_state_space_padded_rows_{self.suffix}")
+        np_rows = int(padded(c_i32(n_state)))
+        bc = torch.empty((tokens, groups, 2, np_rows), dtype=torch.float32, device=proj.device)
+        if np_rows != n_state:
+            bc.zero_()
+        dtd = torch.empty((tokens, heads, 2), dtype=torch.float32, device=proj.device)
         # long portions are cut into blocks that run side by side (the same cut for every layer of the step)
         units = chains = block_states = cum = None
         n_units = n_chains = 0
@@ -1281,12 +1291,14 @@ class HipKernels:
             if n_chains:
                 block_states = torch.empty((n_units, heads, n_state, vdim), dtype=torch.float32, device=proj.device)
                 cum = torch.empty((tokens, heads), dtype=torch.float32, device=proj.device)
-        library.call("ssd", _suffix(proj), "nva_state_space", _p(proj), c_i64(stride), _p(conv_out), _p(y_raw), _p(cum), _p(out),
+        library.call("ssd", _suffix(proj), "nva_state_space", _p(proj), c_i64(stride), _p(conv_out), _p(bc), _p(dtd), _p(y_raw),
+                     _p(cum), _p(out),
                      c_i64(os_), _p(ssm_state), _p(conv_state), c_i64(ssm_state.shape[0]), _p(batch.token_seq),
                      _p(batch.cu_seqlens_q), _p(batch.seq_starts), _p(batch.state_slots), c_i64(seqs), c_i64(tokens),
                      c_i64(first), c_i32(heads), c_i32(vdim), c_i32(n_state), c_i32(groups), c_i32(taps), _p(conv_w),
                      _p(conv_b), _p(dt_bias), _p(a_log), _p(d_skip), _p(norm_w), c_i32(norm_groups), c_f32(eps), _p(units),
-                     c_i64(n_units), _p(chains), c_i64(n_chains), _p(block_states), self._stream())
+                     c_i64(n_units), _p(chains), c_i64(n_chains), _p(block_states), c_i32(self.state_space_shape),
+                     self._stream())
         return out
 
     # ------------------------------------------------------------------ retention
