@@ -78,15 +78,9 @@ def mafarax_config(width: int, layers: int, dtype: str) -> dict:
     value sizes, chunks of 1024 positions, half the head rotated), the state-space half with twice the width in
     heads of 64 channels and 128 state rows, 32 experts of an eighth of the dense inner size of which a token
     runs 6, chosen among 4 of 8 groups, and a shared expert of a quarter of it."""
+    from nano_vllm_amd.models.shapes import _mafarax
     heads, kv, dim, inner = DESIGN_SIZES[width]
-    layer = {"type": "parallel",
-             "mixer": {"left": {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
-                                "mask": {"size": 1024}, "rot": {"dims": dim // 2, "base": 5e5, "scaling": {"factor": 2.0}}},
-                       "right": {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 1}},
-             "mlp": {"kind": "moe", "expert": {"ff": inner // 8}, "shared": {"ff": inner // 4},
-                     "router": {"experts": 32, "top": 6, "scale": 1.0, "groups": {"count": 8, "keep": 4}}}}
-    return {"architecture": "Mafarax", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 1.0,
-            "layers": [layer] * layers, "torch_dtype": dtype}
+    return _mafarax(layers, width, heads, kv, dim, dim, inner, DESIGN_VOCAB, chunk=1024, dtype=dtype)
 
 
 def design_configs(width: int, layers: int, dtype: str, design: str = "nozurax"):

@@ -25,7 +25,7 @@
 #include "common.h"
 
 #define SSD_MAX_TAPS 16
-#define SSD_CONV_TOKENS 8 // tokens in a row that a thread of the convolution takes
+#define SSD_CONV_TOKENS 8 // tokens in a row that a thread of the convolution takes, in steps of many tokens
 #define SSD_TB 16          // tokens whose inputs the recurrence stages at a time
 
 __device__ __forceinline__ float ssd_silu(float x) { return x / (1.f + expf(-x)); }
@@ -39,10 +39,11 @@ ssd_conv_kernel(const T* __restrict__ proj, int64_t stride, int col0, int channe
                 const int32_t* __restrict__ token_seq, const int32_t* __restrict__ cu_seqlens,
                 const int32_t* __restrict__ seq_starts, const int32_t* __restrict__ state_slots,
                 T* __restrict__ out, float* __restrict__ bc, int np, int n_state, int groups, float* __restrict__ dtd,
-                int heads, int dt_col, const float* __restrict__ dt_bias, const float* __restrict__ a_log, int64_t tokens) {
+                int heads, int dt_col, const float* __restrict__ dt_bias, const float* __restrict__ a_log, int64_t tokens,
+                int per_thread) {
     const int c = blockIdx.y * blockDim.x + threadIdx.x;
     if (c >= channels) return;
-    // a thread takes SSD_CONV_TOKENS tokens in a row with its channel's weights in registers
+    // a thread takes per_thread tokens in a row with its channel's weights in registers
     float wt[SSD_MAX_TAPS];
 #pragma unroll
     for (int j = 0; j < SSD_MAX_TAPS; ++j)
@@ -50,7 +51,7 @@ ssd_conv_kernel(const T* __restrict__ proj, int64_t stride, int col0, int channe
     const float bias_c = to_float(conv_b[c]);
     const int hist = taps - 1;
     const int inner = channels - 2 * groups * n_state;
-    for (int64_t t = (int64_t)blockIdx.x * SSD_CONV_TOKENS; t < min(tokens, ((int64_t)blockIdx.x + 1) * SSD_CONV_TOKENS); ++t) {
+    for (int64_t t = (int64_t)blockIdx.x * per_thread; t < min(tokens, ((int64_t)blockIdx.x + 1) * per_thread); ++t) {
         const int s = token_seq[t];
         const int begin = cu_seqlens[s], n = cu_seqlens[s + 1] - begin;
         const int i = (int)(t - begin);                      // the token's place in its request's portion
@@ -369,11 +370,12 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
     if (n_chains && (!units || !chains || !block_states || !cum)) return nva_fail("state_space: blocks need their scratch");
     const elem_t* pj = (const elem_t*)proj;
     if (tokens > 0x7fffffff || (channels + 255) / 256 > 65535) return nva_fail("state_space: too many tokens or channels");
+    const int per_thread = tokens >= 1024 ? SSD_CONV_TOKENS : 1;
     hipLaunchKernelGGL((ssd_conv_kernel<elem_t>),
-                       dim3((unsigned)((tokens + SSD_CONV_TOKENS - 1) / SSD_CONV_TOKENS), (channels + 255) / 256), dim3(256), 0, stream, pj,
+                       dim3((unsigned)((tokens + per_thread - 1) / per_thread), (channels + 255) / 256), dim3(256), 0, stream, pj,
                        stride, inner, channels, taps, (const elem_t*)conv_w, (const elem_t*)conv_b, conv_state, token_seq,
                        cu_seqlens, seq_starts, state_slots, (elem_t*)conv_out, bc, ssd_padded_rows(n_state), n_state, groups, dtd,
-                       heads, inner + channels, dt_bias, a_log, tokens);
+                       heads, inner + channels, dt_bias, a_log, tokens, per_thread);
     if (seqs > num_single && taps > 1)
         hipLaunchKernelGGL((ssd_conv_state_kernel<elem_t>), dim3((channels + 255) / 256, (unsigned)(seqs - num_single)),
                            dim3(256), 0, stream, pj, stride, inner, channels, taps, conv_state, cu_seqlens, seq_starts,

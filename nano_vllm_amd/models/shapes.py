@@ -1,6 +1,7 @@
 """Named config.json contents for runs with random weights (there is no checkpoint to read
-them from): two tiny test shapes and the Qwen3 dense sizes that the benchmarks use, and three
-Nozurax shapes (a tiny one, and layers of the Qwen3 1.7B and 8B sizes).  These are
+them from): two tiny test shapes and the Qwen3 dense sizes that the benchmarks use, three
+Nozurax shapes (a tiny one, and layers of the Qwen3 1.7B and 8B sizes) and two Mafarax shapes (a tiny
+one, and layers of the Qwen3 1.7B sizes).  These are
 inputs, as a model folder's config.json is; nothing in the model code reads them.
 
     python -m nano_vllm_amd.cli random-model --shape qwen3-8b --config-only --out DIR
@@ -38,7 +39,29 @@ def _nozurax(layers, width, heads, kv_heads, dim, vdim, inner, vocab, eps=1e-6, 
             "layers": [kinds[pattern[i % len(pattern)]] for i in range(layers)], "torch_dtype": dtype}
 
 
+def _mafarax(layers, width, heads, kv_heads, dim, vdim, inner, vocab, chunk, eps=1e-6, dtype="bfloat16", rot=None,
+             factor=2.0, ssm_heads=None, ssm_vdim=64, state=128, groups=8, conv=4, norm_groups=1, experts=32, top=6,
+             group_count=8, group_keep=4, logit_scale=1.0) -> dict:
+    """Layers of a chunked attention and a state-space layer side by side and a routed feed-forward: `top` of
+    `experts` experts of inner / 8 each and a shared expert of inner / 4 (a token runs the dense layer's inner size)."""
+    layer = {"type": "parallel",
+             "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
+                                "mask": {"size": chunk},
+                                "rot": {"dims": rot or dim // 2, "base": 5e5, "scaling": {"factor": factor}}},
+                       "right": {"heads": ssm_heads or 2 * width // ssm_vdim, "vdim": ssm_vdim, "state": state,
+                                 "groups": groups, "conv": conv, "norm_groups": norm_groups}},
+             "mlp": {"kind": "moe", "expert": {"ff": max(1, inner // 8)}, "shared": {"ff": max(1, inner // 4)},
+                     "router": {"experts": experts, "top": top, "scale": 1.0,
+                                "groups": {"count": group_count, "keep": group_keep}}}}
+    return {"architecture": "Mafarax", "vocab": vocab, "width": width, "norm": {"eps": eps}, "logit_scale": logit_scale,
+            "layers": [layer] * layers, "torch_dtype": dtype}
+
+
 SHAPES: Dict[str, dict] = {
+    "mafarax-tiny": _mafarax(3, 64, 4, 2, 16, 24, 96, 256, chunk=12, eps=1e-5, dtype="float32", rot=8, ssm_heads=4,
+                             ssm_vdim=8, state=12, groups=2, conv=3, norm_groups=2, experts=6, top=2, group_count=3,
+                             group_keep=2, logit_scale=1.5),
+    "mafarax-1b": _mafarax(16, 2048, 16, 8, 128, 128, 6144, 32768, chunk=1024),
     "nozurax-tiny": _nozurax(4, 64, 4, 2, 16, 24, 96, 256, eps=1e-5, every=8, dtype="float32", ret_heads=2, rot=8),
     "nozurax-1b": _nozurax(16, 2048, 16, 8, 128, 128, 6144, 32768),
     "nozurax-8b": _nozurax(32, 4096, 32, 8, 128, 128, 12288, 32768),
