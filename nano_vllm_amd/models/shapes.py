@@ -40,14 +40,14 @@ def _nozurax(layers, width, heads, kv_heads, dim, vdim, inner, vocab, eps=1e-6, 
 
 
 def _mafarax(layers, width, heads, kv_heads, dim, vdim, inner, vocab, chunk, eps=1e-6, dtype="bfloat16", rot=None,
-             factor=2.0, ssm_heads=None, ssm_vdim=64, state=128, groups=8, conv=4, norm_groups=1, experts=32, top=6,
+             factor=4.0, ssm_heads=None, ssm_vdim=64, state=128, groups=8, conv=4, norm_groups=1, experts=32, top=6,
              group_count=8, group_keep=4, logit_scale=1.0) -> dict:
     """Layers of a chunked attention and a state-space layer side by side and a routed feed-forward: `top` of
     `experts` experts of inner / 8 each and a shared expert of inner / 4 (a token runs the dense layer's inner size)."""
     layer = {"type": "parallel",
              "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
                                 "mask": {"size": chunk},
-                                "rot": {"dims": rot or dim // 2, "base": 5e5, "scaling": {"factor": factor}}},
+                                "rot": {"dims": rot or dim // 2, "base": 1e6, "scaling": {"factor": factor}}},
                        "right": {"heads": ssm_heads or 2 * width // ssm_vdim, "vdim": ssm_vdim, "state": state,
                                  "groups": groups, "conv": conv, "norm_groups": norm_groups}},
              "mlp": {"kind": "moe", "expert": {"ff": max(1, inner // 8)}, "shared": {"ff": max(1, inner // 4)},

@@ -39,16 +39,16 @@ CONFIGS: Dict[str, dict] = {
         page=8, seed=31),
     # sizes of the matrix-core kernels' kind (equal head sizes of 64, multiples of 32 everywhere)
     "b": dict(cfg=MafaraxConfig(vocab=512, width=128, eps=1e-6, logit_scale=3.0, layers=(
-        MafaraxLayer(Att(8, 2, 64, 64, 0.11, 48, rot_dims=32, rot_base=5e5, rot_factor=2.0),
+        MafaraxLayer(Att(8, 2, 64, 64, 0.11, 48, rot_dims=32, rot_base=2e5, rot_factor=3.0),
                      Ssm(heads=4, vdim=64, state=64, groups=2, conv=4, norm_groups=2),
                      Moe(experts=8, top=3, ff=64, scale=0.7, group_count=4, group_keep=2, shared_ff=96)),
-        MafaraxLayer(Att(8, 2, 64, 64, 0.11, 48, rot_dims=32, rot_base=5e5, rot_factor=2.0),
+        MafaraxLayer(Att(8, 2, 64, 64, 0.11, 48, rot_dims=32, rot_base=2e5, rot_factor=3.0),
                      Ssm(heads=4, vdim=64, state=64, groups=2, conv=4, norm_groups=2),
                      Moe(experts=8, top=3, ff=64, scale=0.7, group_count=4, group_keep=2, shared_ff=96)))),
         page=32, seed=32),
     "c": dict(cfg=MafaraxConfig(vocab=97, width=20, eps=1e-6, logit_scale=1.0, layers=(
         MafaraxLayer(Att(3, 3, 6, 10, 0.4, 1), Ssm(heads=2, vdim=5, state=3, groups=2, conv=5, norm_groups=1),
-                     Moe(experts=5, top=3, ff=9, scale=1.5, group_count=5, group_keep=3, shared_ff=7)),
+                     Moe(experts=5, top=3, ff=9, scale=1.3, group_count=5, group_keep=3, shared_ff=7)),
         MafaraxLayer(Att(3, 1, 8, 4, 0.5, 4096, rot_dims=6, rot_base=50.0, rot_factor=1.5),
                      Ssm(heads=1, vdim=20, state=40, groups=1, conv=4, norm_groups=4),
                      Moe(experts=9, top=2, ff=6, scale=0.9, group_count=3, group_keep=1, shared_ff=11)))),
@@ -56,7 +56,7 @@ CONFIGS: Dict[str, dict] = {
     "d": dict(cfg=MafaraxConfig(vocab=333, width=72, eps=1e-6, logit_scale=1.25, layers=(
         MafaraxLayer(Att(6, 2, 24, 40, 0.25, 33, rot_dims=24, rot_base=1e6, rot_factor=8.0),
                      Ssm(heads=6, vdim=12, state=16, groups=3, conv=4, norm_groups=2),
-                     Moe(experts=12, top=2, ff=30, scale=1.0, group_count=4, group_keep=2, shared_ff=30)),)),
+                     Moe(experts=15, top=2, ff=30, scale=1.0, group_count=5, group_keep=2, shared_ff=30)),)),
         page=16, seed=34),
 }
 
