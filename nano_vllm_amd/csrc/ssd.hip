@@ -202,14 +202,35 @@ ssd_scan_kernel(const T* __restrict__ conv, int channels, const float* __restric
         const int nb = min(SSD_TB, n - i0);
         const int64_t tb = t0 + i0;
         __syncthreads();
-        if (!SC)
-            for (int idx = lane; idx < nb * NMAX; idx += NVA_WAVE) {          // (np == NMAX here)
-                const int j = idx / NMAX, k = idx % NMAX;
-                c_s[j][k] = bc_g[(tb + j) * bc_stride + np + k];
-                if (mode != 2) b_s[j][k] = bc_g[(tb + j) * bc_stride + k];
-            }
-        if (mode != 2)
-            for (int j = 0; j < nb; ++j) x_s[j][lane] = mine ? to_float(conv[(tb + j) * channels + h * vdim + p]) : 0.f;   // (a column's lanes hold the same)
+        // (every load of a batch is asked for before any is used: a loop of load and store would wait for each in turn)
+        if (!SC) {
+            // a token's B and C lie side by side in bc, 2 np floats: the wave copies them 16 bytes a lane (np == NMAX here)
+            constexpr int PER = 2 * NMAX / 4 / NVA_WAVE > 0 ? 2 * NMAX / 4 / NVA_WAVE : 1;     // float4 a lane and token
+            float4 v[SSD_TB][PER];
+#pragma unroll
+            for (int j = 0; j < SSD_TB; ++j)
+#pragma unroll
+                for (int q = 0; q < PER; ++q) {
+                    const int at = (q * NVA_WAVE + lane) * 4;
+                    v[j][q] = j < nb && at < 2 * NMAX ? *reinterpret_cast<const float4*>(bc_g + (tb + j) * bc_stride + at)
+                                                      : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+#pragma unroll
+            for (int j = 0; j < SSD_TB; ++j)
+#pragma unroll
+                for (int q = 0; q < PER; ++q) {
+                    const int at = (q * NVA_WAVE + lane) * 4;
+                    if (at < NMAX) *reinterpret_cast<float4*>(&b_s[j][at]) = v[j][q];
+                    else if (at < 2 * NMAX) *reinterpret_cast<float4*>(&c_s[j][at - NMAX]) = v[j][q];
+                }
+        }
+        if (mode != 2) {
+            float xv[SSD_TB];
+#pragma unroll
+            for (int j = 0; j < SSD_TB; ++j) xv[j] = j < nb && mine ? to_float(conv[(tb + j) * channels + h * vdim + p]) : 0.f;
+#pragma unroll
+            for (int j = 0; j < SSD_TB; ++j) x_s[j][lane] = xv[j];          // (a column's lanes hold the same)
+        }
         __syncthreads();
         auto step = [&](int j) __attribute__((always_inline)) {
             const int64_t t = tb + j;
@@ -289,6 +310,78 @@ ssd_chain_kernel(float* __restrict__ block_states, const float* __restrict__ cum
     state[((int64_t)state_slots[s] * heads + h) * per_head + e] = carry;
 }
 
+// ---------------------------------------------------------------------------- what the state before a block adds
+// y[t, p] += exp(cum[t]) * sum_n C[t, n] E[n, p] for the tokens t of a block, E the true state before the block: one float
+// product per block and head, on the matrix cores (v_mfma_f32_32x32x2_f32: float operands, float sums).  A workgroup of
+// four waves takes 64 tokens of a block and 64 columns; C of those tokens and the 64 columns of E are staged in LDS (rows
+// beyond the state's are zero there).
+typedef __attribute__((ext_vector_type(16))) float ssd_f32x16;
+
+__global__ void __launch_bounds__(256)
+ssd_inter_kernel(const float* __restrict__ bc, int np, int heads, int vdim, int n_state, int groups,
+                 const int32_t* __restrict__ cu_seqlens, int first_seq, const int32_t* __restrict__ units, int subs,
+                 const float* __restrict__ block_states, const float* __restrict__ cum, float* __restrict__ y) {
+    extern __shared__ __attribute__((aligned(16))) float c_lds[];          // [64 tokens][kp + 1], then E [kp][64]
+    const int u = blockIdx.z / subs, sub = blockIdx.z % subs, h = blockIdx.y;
+    if (units[4 * u + 1] == 0) return;                                      // a portion's first block started from the true state
+    const int n = units[4 * u + 2];
+    const int i0 = sub * 64;
+    if (i0 >= n) return;
+    const int64_t t0 = cu_seqlens[first_seq + units[4 * u]] + units[4 * u + 1] + i0;
+    const int rows = min(64, n - i0);
+    const int kp = (n_state + 1) & ~1;                                      // k in pairs
+    const int ld = kp + 1;
+    const int g = h / (heads / groups);
+    const int64_t bc_stride = (int64_t)groups * 2 * np;
+    const float* c_g = bc + (int64_t)g * 2 * np + np;
+    float* e_lds = c_lds + 64 * ld;
+    const float* e = block_states + (((int64_t)(u - 1) * heads + h) * n_state) * vdim;
+    const int pw = blockIdx.x * 64;                                        // the workgroup's first column
+    // (eight loads asked for before any is used: a loop of load and store would wait for each in turn)
+    for (int base = 0; base < 64 * kp; base += 8 * 256) {
+        float vc[8], ve[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const int idx = base + q * 256 + threadIdx.x;
+            const int r = idx / kp, k = idx % kp;                           // C: token r, row k
+            vc[q] = idx < 64 * kp && r < rows && k < n_state ? c_g[(t0 + r) * bc_stride + k] : 0.f;
+            const int ke = idx / 64, j = idx % 64;                          // E: row ke, column j
+            ve[q] = idx < 64 * kp && ke < n_state && pw + j < vdim ? e[(int64_t)ke * vdim + pw + j] : 0.f;
+        }
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const int idx = base + q * 256 + threadIdx.x;
+            if (idx < 64 * kp) {
+                c_lds[(idx / kp) * ld + idx % kp] = vc[q];
+                e_lds[idx] = ve[q];
+            }
+        }
+    }
+    __syncthreads();
+    const int wave = threadIdx.x / NVA_WAVE, lane = threadIdx.x % NVA_WAVE;
+    const int tt = wave / 2, p0 = blockIdx.x * 64 + (wave % 2) * 32;
+    if (tt * 32 >= rows || p0 >= vdim) return;
+    const int i = lane % 32, half = lane / 32;
+    const int inner = heads * vdim;
+    const bool col_ok = p0 + i < vdim;
+    ssd_f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    const float* crow = c_lds + (tt * 32 + i) * ld + half;
+    const float* ecol = e_lds + half * 64 + (wave % 2) * 32 + i;
+#pragma unroll 8
+    for (int k = 0; k < kp; k += 2) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(crow[k], ecol[k * 64], acc, 0, 0, 0);
+    // acc[r] is the sum of row 8 (r / 4) + 4 half + r % 4, column i
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int row = tt * 32 + 8 * (r / 4) + 4 * half + r % 4;
+        if (row < rows && col_ok) {
+            const int64_t t = t0 + row;
+            y[t * inner + h * vdim + p0 + i] += expf(cum[t * heads + h]) * acc[r];
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------- gate and grouped norm
 template <typename T>
 __global__ void __launch_bounds__(1024)
@@ -338,8 +431,8 @@ static void launch_scan(const ScanArgs& a, unsigned units, int first_seq, const 
 // and cum [tokens, H] (float) are scratch.  state [slots, H, N, P], conv_state [slots, C, K - 1], float.
 // The first num_single requests bring one token each.  units / chains (with block_states [units, H, N, P]): the
 // portions of the requests from num_single on cut into blocks (units[u] = request counted from num_single, first token,
-// tokens, blocks of the portion; shape: 0, or how a state of 65 to 128 rows is held (1: a thread a column, 2: four
-// lanes a column; measurements); chains[c] = first unit, blocks, request, tokens of the last block, for every
+// tokens, blocks of the portion; block_tokens: the most tokens of a block; shape: 0, or how a state of 65 to 128 rows is held (1: a thread a column, 2: four
+// lanes a column, 3: the second pass on the vector units; measurements); chains[c] = first unit, blocks, request, tokens of the last block, for every
 // portion of more than one block); null: every portion runs as one.
 // bc: float [tokens, groups, 2, padded rows] (zero where the padded rows exceed the state's: the caller clears it then),
 // dtd: float [tokens, heads, 2]: scratch as well.
@@ -351,8 +444,8 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
                                          int heads, int vdim, int n_state, int groups, int taps, const void* conv_w,
                                          const void* conv_b, const float* dt_bias, const float* a_log, const float* d_skip,
                                          const float* norm_w, int norm_groups, float eps, const int32_t* units,
-                                         int64_t n_units, const int32_t* chains, int64_t n_chains, float* block_states,
-                                         int shape, hipStream_t stream) {
+                                         int64_t n_units, const int32_t* chains, int64_t n_chains, int block_tokens,
+                                         float* block_states, int shape, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || seqs <= 0 || seqs > 65535 || num_single < 0 || num_single > seqs || slots <= 0)
         return nva_fail("state_space: bad counts tokens=%lld requests=%lld", (long long)tokens, (long long)seqs);
@@ -367,7 +460,8 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
     if (!proj || !conv_out || !bc || !dtd || !y_raw || !out || !state || (!conv_state && taps > 1) || !token_seq || !cu_seqlens || !seq_starts ||
         !state_slots || !conv_w || !conv_b || !dt_bias || !a_log || !d_skip || !norm_w)
         return nva_fail("state_space: a tensor is missing");
-    if (n_chains && (!units || !chains || !block_states || !cum)) return nva_fail("state_space: blocks need their scratch");
+    if (n_chains && (!units || !chains || !block_states || !cum || block_tokens <= 0 || n_units * ((block_tokens + 63) / 64) > 65535))
+        return nva_fail("state_space: blocks need their scratch and their size");
     const elem_t* pj = (const elem_t*)proj;
     if (tokens > 0x7fffffff || (channels + 255) / 256 > 65535) return nva_fail("state_space: too many tokens or channels");
     const int per_thread = tokens >= 1024 ? SSD_CONV_TOKENS : 1;
@@ -399,7 +493,23 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
         hipLaunchKernelGGL(ssd_chain_kernel, dim3((n_state * vdim + 255) / 256, heads, (unsigned)n_chains), dim3(256), 0, stream,
                            block_states, cum, state, chains, units, cu_seqlens, state_slots, (int)num_single, heads, n_state,
                            vdim);
-        scan((unsigned)n_units, (int)num_single, units, 2);
+        if (shape == 3) {
+            scan((unsigned)n_units, (int)num_single, units, 2);              // (on the vector units: measurements)
+        } else {
+            // the blocks' tokens: `block_tokens` at most, 64 a workgroup
+            const int subs = (block_tokens + 63) / 64;
+            const int kp = (n_state + 1) & ~1;
+            static bool raised = false;              // the kernel's LDS limit, lifted once to what the tallest state needs
+            if (!raised) {
+                if (hipFuncSetAttribute((const void*)ssd_inter_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)((64 * 257 + 256 * 64) * sizeof(float))) != hipSuccess)
+                    return nva_fail("state_space: cannot have the LDS of the blocks' second pass");
+                raised = true;
+            }
+            hipLaunchKernelGGL(ssd_inter_kernel, dim3((unsigned)((vdim + 63) / 64), (unsigned)heads, (unsigned)(n_units * subs)),
+                               dim3(256), (size_t)(64 * (kp + 1) + kp * 64) * sizeof(float), stream, bc, ssd_padded_rows(n_state), heads, vdim,
+                               n_state, groups, cu_seqlens, (int)num_single, units, subs, block_states, cum, y_raw);
+        }
     } else {
         scan((unsigned)seqs, 0, nullptr, 0);
     }

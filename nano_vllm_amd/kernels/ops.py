@@ -1272,7 +1272,7 @@ class HipKernels:
         dtd = torch.empty((tokens, heads, 2), dtype=torch.float32, device=proj.device)
         # long portions are cut into blocks that run side by side (the same cut for every layer of the step)
         units = chains = block_states = cum = None
-        n_units = n_chains = 0
+        n_units = n_chains = block_tokens = 0
         first = batch.num_decode
         if self.state_space_blocks_side_by_side and first < seqs:
             kept = getattr(batch, "step_cache", None)
@@ -1280,14 +1280,15 @@ class HipKernels:
                 kept = batch.step_cache = {}
             plan = kept.get(("state_space_blocks", first))
             if plan is None:
-                _, flat_units, flat_chains = retention_blocks(batch.q_lens, first)
+                block_tokens, flat_units, flat_chains = retention_blocks(batch.q_lens, first)
                 if flat_chains:
                     both = torch.tensor(flat_units + flat_chains, dtype=torch.int32).to(proj.device, non_blocking=True)
-                    plan = (len(flat_units) // 4, len(flat_chains) // 4, both[: len(flat_units)], both[len(flat_units):])
+                    plan = (len(flat_units) // 4, len(flat_chains) // 4, both[: len(flat_units)], both[len(flat_units):],
+                            block_tokens)
                 else:
-                    plan = (0, 0, None, None)
+                    plan = (0, 0, None, None, 0)
                 kept[("state_space_blocks", first)] = plan
-            n_units, n_chains, units, chains = plan
+            n_units, n_chains, units, chains, block_tokens = plan
             if n_chains:
                 block_states = torch.empty((n_units, heads, n_state, vdim), dtype=torch.float32, device=proj.device)
                 cum = torch.empty((tokens, heads), dtype=torch.float32, device=proj.device)
@@ -1297,7 +1298,8 @@ class HipKernels:
                      _p(batch.cu_seqlens_q), _p(batch.seq_starts), _p(batch.state_slots), c_i64(seqs), c_i64(tokens),
                      c_i64(first), c_i32(heads), c_i32(vdim), c_i32(n_state), c_i32(groups), c_i32(taps), _p(conv_w),
                      _p(conv_b), _p(dt_bias), _p(a_log), _p(d_skip), _p(norm_w), c_i32(norm_groups), c_f32(eps), _p(units),
-                     c_i64(n_units), _p(chains), c_i64(n_chains), _p(block_states), c_i32(self.state_space_shape),
+                     c_i64(n_units), _p(chains), c_i64(n_chains), c_i32(block_tokens), _p(block_states),
+                     c_i32(self.state_space_shape),
                      self._stream())
         return out
 
