@@ -216,20 +216,23 @@ ssd_scan_kernel(const T* __restrict__ conv, int channels, const float* __restric
                                                       : make_float4(0.f, 0.f, 0.f, 0.f);
                 }
 #pragma unroll
-            for (int j = 0; j < SSD_TB; ++j)
+            for (int j = 0; j < SSD_TB; ++j) {
+                if (j >= nb) break;
 #pragma unroll
                 for (int q = 0; q < PER; ++q) {
                     const int at = (q * NVA_WAVE + lane) * 4;
                     if (at < NMAX) *reinterpret_cast<float4*>(&b_s[j][at]) = v[j][q];
                     else if (at < 2 * NMAX) *reinterpret_cast<float4*>(&c_s[j][at - NMAX]) = v[j][q];
                 }
+            }
         }
         if (mode != 2) {
             float xv[SSD_TB];
 #pragma unroll
             for (int j = 0; j < SSD_TB; ++j) xv[j] = j < nb && mine ? to_float(conv[(tb + j) * channels + h * vdim + p]) : 0.f;
 #pragma unroll
-            for (int j = 0; j < SSD_TB; ++j) x_s[j][lane] = xv[j];          // (a column's lanes hold the same)
+            for (int j = 0; j < SSD_TB; ++j)
+                if (j < nb) x_s[j][lane] = xv[j];                            // (a column's lanes hold the same)
         }
         __syncthreads();
         auto step = [&](int j) __attribute__((always_inline)) {
