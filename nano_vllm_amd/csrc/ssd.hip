@@ -313,6 +313,58 @@ ssd_chain_kernel(float* __restrict__ block_states, const float* __restrict__ cum
     state[((int64_t)state_slots[s] * heads + h) * per_head + e] = carry;
 }
 
+// ---------------------------------------------------------------------------- single tokens
+// A request that brings one token: the step is the state's bytes, read once and written once.  A workgroup of four
+// waves takes (request, head, 64 columns of S); a thread one column and every fourth row, all of its rows asked
+// for before B, C and the step size arrive; the four partial read-outs of a column meet in LDS.
+__global__ void __launch_bounds__(256)
+ssd_single_kernel(const void* __restrict__ conv, int conv_is_f32, int channels, const float* __restrict__ bc, int np,
+                  const float* __restrict__ dtd, int heads, int vdim, int n_state, int groups,
+                  const float* __restrict__ d_skip, float* __restrict__ state, const int32_t* __restrict__ cu_seqlens,
+                  const int32_t* __restrict__ seq_starts, const int32_t* __restrict__ state_slots,
+                  float* __restrict__ y) {
+    __shared__ float b_s[256], c_s[256], part_s[4][64];
+    const int s = blockIdx.z, h = blockIdx.y;
+    const int pl = threadIdx.x % 64, rg = threadIdx.x / 64;
+    const int p = blockIdx.x * 64 + pl;
+    const bool mine = p < vdim;
+    const int64_t t = cu_seqlens[s];
+    const bool carried = seq_starts[s] > 0;
+    float* own = state + (((int64_t)state_slots[s] * heads + h) * n_state) * vdim + p;
+    constexpr int ROWS = 64;                          // rows of a thread: every fourth of up to 256
+    float S[ROWS];
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        const int r = rg + 4 * i;
+        S[i] = carried && mine && r < n_state ? own[(int64_t)r * vdim] : 0.f;
+    }
+    const int g = h / (heads / groups);
+    const float* bt = bc + (t * groups + g) * 2 * (int64_t)np;
+    for (int k = threadIdx.x; k < n_state; k += 256) {
+        b_s[k] = bt[k];
+        c_s[k] = bt[np + k];
+    }
+    const float dt = dtd[(t * heads + h) * 2], decay = dtd[(t * heads + h) * 2 + 1];
+    const int64_t xi = t * channels + h * vdim + p;
+    const float x = !mine ? 0.f : conv_is_f32 ? static_cast<const float*>(conv)[xi] : to_float(static_cast<const __bf16*>(conv)[xi]);
+    __syncthreads();
+    const float dx = dt * x;
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        const int r = rg + 4 * i;
+        if (r < n_state) {
+            S[i] = decay * S[i] + b_s[r] * dx;
+            acc += S[i] * c_s[r];
+            if (mine) own[(int64_t)r * vdim] = S[i];
+        }
+    }
+    part_s[rg][pl] = acc;
+    __syncthreads();
+    if (rg == 0 && mine)
+        y[t * heads * vdim + h * vdim + p] = part_s[0][pl] + part_s[1][pl] + part_s[2][pl] + part_s[3][pl] + d_skip[h] * x;
+}
+
 // ---------------------------------------------------------------------------- what the state before a block adds
 // y[t, p] += exp(cum[t]) * sum_n C[t, n] E[n, p] for the tokens t of a block, E the true state before the block: one float
 // product per block and head, on the matrix cores (v_mfma_f32_32x32x2_f32: float operands, float sums).  A workgroup of
@@ -435,7 +487,8 @@ static void launch_scan(const ScanArgs& a, unsigned units, int first_seq, const 
 // The first num_single requests bring one token each.  units / chains (with block_states [units, H, N, P]): the
 // portions of the requests from num_single on cut into blocks (units[u] = request counted from num_single, first token,
 // tokens, blocks of the portion; block_tokens: the most tokens of a block; shape: 0, or how a state of 65 to 128 rows is held (1: a thread a column, 2: four
-// lanes a column, 3: the second pass on the vector units; measurements); chains[c] = first unit, blocks, request, tokens of the last block, for every
+// lanes a column, 3: the second pass on the vector units, 4: single
+// tokens through the kernel that serves portions; measurements); chains[c] = first unit, blocks, request, tokens of the last block, for every
 // portion of more than one block); null: every portion runs as one.
 // bc: float [tokens, groups, 2, padded rows] (zero where the padded rows exceed the state's: the caller clears it then),
 // dtd: float [tokens, heads, 2]: scratch as well.
@@ -489,9 +542,18 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
         else if (n_state <= 128) launch_scan<64, 2>(args, units, first_seq, us, mode, stream);
         else launch_scan<64, 4>(args, units, first_seq, us, mode, stream);
     };
+    // the requests that bring one token (they come first) have a kernel of their own
+    auto single = [&]() {
+        if (num_single && shape != 4)
+            hipLaunchKernelGGL(ssd_single_kernel, dim3((unsigned)((vdim + 63) / 64), (unsigned)heads, (unsigned)num_single), dim3(256),
+                               0, stream, conv_out, (int)(sizeof(elem_t) == 4), channels, bc, ssd_padded_rows(n_state), dtd, heads,
+                               vdim, n_state, groups, d_skip, state, cu_seqlens, seq_starts, state_slots, y_raw);
+        else if (num_single)
+            scan((unsigned)num_single, 0, nullptr, 0);
+    };
     if (n_chains) {
         if (n_units <= 0 || n_units > 65535) return nva_fail("state_space: bad block count %lld", (long long)n_units);
-        if (num_single) scan((unsigned)num_single, 0, nullptr, 0);
+        single();
         scan((unsigned)n_units, (int)num_single, units, 1);
         hipLaunchKernelGGL(ssd_chain_kernel, dim3((n_state * vdim + 255) / 256, heads, (unsigned)n_chains), dim3(256), 0, stream,
                            block_states, cum, state, chains, units, cu_seqlens, state_slots, (int)num_single, heads, n_state,
@@ -514,7 +576,11 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
                                n_state, groups, cu_seqlens, (int)num_single, units, subs, block_states, cum, y_raw);
         }
     } else {
-        scan((unsigned)seqs, 0, nullptr, 0);
+        single();
+        if (seqs > num_single) {
+            // (units == null: unit u is request first_seq + u)
+            scan((unsigned)(seqs - num_single), (int)num_single, nullptr, 0);
+        }
     }
     const int group_size = inner / norm_groups;
     // (few tokens: more threads a row, so that a row's loads are on their way at once)
