@@ -215,24 +215,23 @@ ssd_scan_kernel(const T* __restrict__ conv, int channels, const float* __restric
                     v[j][q] = j < nb && at < 2 * NMAX ? *reinterpret_cast<const float4*>(bc_g + (tb + j) * bc_stride + at)
                                                       : make_float4(0.f, 0.f, 0.f, 0.f);
                 }
+            // (rows of a short batch beyond its tokens are written too, as zeros: a store behind a branch would hold up
+            // the others)
 #pragma unroll
-            for (int j = 0; j < SSD_TB; ++j) {
-                if (j >= nb) break;
+            for (int j = 0; j < SSD_TB; ++j)
 #pragma unroll
                 for (int q = 0; q < PER; ++q) {
                     const int at = (q * NVA_WAVE + lane) * 4;
                     if (at < NMAX) *reinterpret_cast<float4*>(&b_s[j][at]) = v[j][q];
                     else if (at < 2 * NMAX) *reinterpret_cast<float4*>(&c_s[j][at - NMAX]) = v[j][q];
                 }
-            }
         }
         if (mode != 2) {
             float xv[SSD_TB];
 #pragma unroll
             for (int j = 0; j < SSD_TB; ++j) xv[j] = j < nb && mine ? to_float(conv[(tb + j) * channels + h * vdim + p]) : 0.f;
 #pragma unroll
-            for (int j = 0; j < SSD_TB; ++j)
-                if (j < nb) x_s[j][lane] = xv[j];                            // (a column's lanes hold the same)
+            for (int j = 0; j < SSD_TB; ++j) x_s[j][lane] = xv[j];          // (a column's lanes hold the same)
         }
         __syncthreads();
         auto step = [&](int j) __attribute__((always_inline)) {
