@@ -148,7 +148,7 @@ ssd_scan_kernel(const T* __restrict__ conv, int channels, const float* __restric
                 const float* __restrict__ a_log, const float* __restrict__ d_skip, float* __restrict__ state,
                 const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_starts,
                 const int32_t* __restrict__ state_slots, int first_seq, const int32_t* __restrict__ units, int mode,
-                float* __restrict__ block_states, float* __restrict__ cum, float* __restrict__ y) {
+                int carried_only, float* __restrict__ block_states, float* __restrict__ cum, float* __restrict__ y) {
     // B, C, x, the step size and the decay of SSD_TB tokens at a time: their loads are on their way
     // together, and the tokens of a batch run from LDS
     constexpr bool SC = NSPLIT == 1;
@@ -172,6 +172,9 @@ ssd_scan_kernel(const T* __restrict__ conv, int channels, const float* __restric
         n = cu_seqlens[s + 1] - t0;
     }
     if (mode == 2 && first_block) return;
+    // (carried_only: the blocks from a zero state have a kernel of their own; this one takes those that go on from
+    // the request's state)
+    if (mode == 1 && carried_only && !(first_block && seq_starts[s] > 0)) return;
     const int inner = heads * vdim;
     const int g = h / (heads / groups);
     const float* bc_g = bc + (int64_t)g * 2 * np;             // token t: + t * groups * 2 * np; C: + np
@@ -364,12 +367,168 @@ ssd_single_kernel(const void* __restrict__ conv, int conv_is_f32, int channels, 
         y[t * heads * vdim + h * vdim + p] = part_s[0][pl] + part_s[1][pl] + part_s[2][pl] + part_s[3][pl] + d_skip[h] * x;
 }
 
+typedef __attribute__((ext_vector_type(16))) float ssd_f32x16;
+
+// ---------------------------------------------------------------------------- a block from a zero state, as products
+// With cum_t the sum of the log-decays of the block's tokens up to t, a block that starts from a zero state gives
+//     y_t = sum over s <= t of exp(cum_t - cum_s) dt_s (C_t . B_s) x_s + D x_t         and leaves
+//     U   = sum over s of exp(cum_last - cum_s) dt_s B_s x_s^T                          as its end state:
+// no recurrence, three float products (C B^T, the masked and weighted result times X, B^T times the weighted X) on
+// the matrix cores (v_mfma_f32_32x32x2_f32).  Every exponent is a difference of sums of logarithms that is <= 0.
+// A workgroup of four waves takes a block of up to 64 tokens, a head and 64 columns; C, B and X are staged in LDS,
+// the masked product goes through LDS to become an operand.  States of up to 128 rows.
+__global__ void __launch_bounds__(256)
+ssd_block_kernel(const void* __restrict__ conv, int conv_is_f32, int channels, const float* __restrict__ bc, int np,
+                 const float* __restrict__ dtd, int heads, int vdim, int n_state, int groups,
+                 const float* __restrict__ a_log, const float* __restrict__ d_skip, float* __restrict__ state,
+                 const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_starts,
+                 const int32_t* __restrict__ state_slots, int first_seq, const int32_t* __restrict__ units,
+                 float* __restrict__ block_states, float* __restrict__ cum, float* __restrict__ y) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int u = blockIdx.z, h = blockIdx.y, pw = blockIdx.x * 64;
+    const int s = first_seq + units[4 * u];
+    const bool first_block = units[4 * u + 1] == 0;
+    if (first_block && seq_starts[s] > 0) return;          // goes on from the request's state: the recurrence's kernel
+    const int n = units[4 * u + 2], blocks = units[4 * u + 3];
+    const int64_t t0 = cu_seqlens[s] + units[4 * u + 1];
+    const int nt = (n_state + 31) / 32;                    // tiles of 32 rows of the state
+    const int ld = 32 * nt + 1;                            // C and B rows in LDS, zero beyond the state's rows
+    float* c_s = lds;                                      // [64][ld]
+    float* b_s = c_s + 64 * ld;                            // [64][ld]
+    float* x_s = b_s + 64 * ld;                            // [64][65]
+    float* m_s = x_s + 64 * 65;                            // [64][65]
+    float* cum_s = m_s + 64 * 65;                          // [64]
+    float* dt_s = cum_s + 64;                              // [64]
+    const int tid = threadIdx.x, wave = tid / NVA_WAVE, lane = tid % NVA_WAVE;
+    const int g = h / (heads / groups);
+    const int64_t bc_stride = (int64_t)groups * 2 * np;
+    const float* bc_g = bc + (int64_t)g * 2 * np;
+    const int width = 32 * nt;
+    // B and C of the block's tokens, 16 bytes a load, every load asked for before any is used (the rows are padded
+    // with zeros up to np in memory; beyond np and beyond the block's tokens zeros are written)
+    {
+        const int w4 = width / 4;                          // float4 a row
+        constexpr int MAXQ = 64 * 32 / 256;                // a row has at most 128 floats
+        float4 vb[MAXQ], vc[MAXQ];
+#pragma unroll
+        for (int q = 0; q < MAXQ; ++q) {
+            const int idx = q * 256 + tid, r = idx / w4, k = (idx % w4) * 4;
+            const bool ok = idx < 64 * w4 && r < n && k < np;
+            vb[q] = ok ? *reinterpret_cast<const float4*>(bc_g + (t0 + r) * bc_stride + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+            vc[q] = ok ? *reinterpret_cast<const float4*>(bc_g + (t0 + r) * bc_stride + np + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int q = 0; q < MAXQ; ++q) {
+            const int idx = q * 256 + tid;
+            if (idx < 64 * w4) {
+                float* bd = b_s + (idx / w4) * ld + (idx % w4) * 4;
+                float* cd = c_s + (idx / w4) * ld + (idx % w4) * 4;
+                bd[0] = vb[q].x, bd[1] = vb[q].y, bd[2] = vb[q].z, bd[3] = vb[q].w;
+                cd[0] = vc[q].x, cd[1] = vc[q].y, cd[2] = vc[q].z, cd[3] = vc[q].w;
+            }
+        }
+    }
+    {
+        float vx[16];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            const int idx = q * 256 + tid, r = idx / 64, j = idx % 64;
+            const int64_t at = (t0 + r) * channels + h * vdim + pw + j;
+            vx[q] = r < n && pw + j < vdim ? (conv_is_f32 ? static_cast<const float*>(conv)[at]
+                                                         : to_float(static_cast<const __bf16*>(conv)[at])) : 0.f;
+        }
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            const int idx = q * 256 + tid;
+            x_s[(idx / 64) * 65 + idx % 64] = vx[q];
+        }
+    }
+    if (wave == 0) {
+        // the tokens' log-decays summed along the block, by one wave
+        const float dt = lane < n ? dtd[((t0 + lane) * heads + h) * 2] : 0.f;
+        float c = -expf(a_log[h]) * dt;
+#pragma unroll
+        for (int off = 1; off < NVA_WAVE; off <<= 1) {
+            const float up = __shfl_up(c, off, NVA_WAVE);
+            if (lane >= off) c += up;
+        }
+        cum_s[lane] = c;
+        dt_s[lane] = dt;
+        if (lane < n && blockIdx.x == 0) cum[(t0 + lane) * heads + h] = c;
+    }
+    __syncthreads();
+    const int i = lane % 32, half = lane / 32;
+    typedef ssd_f32x16 acc_t;
+    // ---- G = C B^T, tile (ti, si) of 32 tokens t by 32 tokens s; then masked and weighted into m_s
+    {
+        const int ti = wave / 2, si = wave % 2;
+        acc_t acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        if (si <= ti) {                                      // (the tile above the diagonal is all zero)
+            const float* crow = c_s + (32 * ti + i) * ld + half;
+            const float* brow = b_s + (32 * si + i) * ld + half;
+#pragma unroll 8
+            for (int k = 0; k < width; k += 2) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(crow[k], brow[k], acc, 0, 0, 0);
+        }
+        const int sc = 32 * si + i;
+        const float cum_sc = cum_s[sc], dt_sc = dt_s[sc];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int t = 32 * ti + 8 * (r / 4) + 4 * half + r % 4;
+            m_s[t * 65 + sc] = sc <= t ? acc[r] * expf(cum_s[t] - cum_sc) * dt_sc : 0.f;
+        }
+    }
+    __syncthreads();
+    const int inner = heads * vdim;
+    // ---- Y = M X, tile (ti, pi) of 32 tokens by 32 columns
+    {
+        const int ti = wave / 2, pi = wave % 2;
+        acc_t acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        const float* mrow = m_s + (32 * ti + i) * 65 + half;
+        const float* xcol = x_s + half * 65 + 32 * pi + i;
+#pragma unroll 8
+        for (int k = 0; k < 32 * (ti + 1); k += 2) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(mrow[k], xcol[k * 65], acc, 0, 0, 0);
+        const float skip = d_skip[h];
+        const int pc = pw + 32 * pi + i;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int t = 32 * ti + 8 * (r / 4) + 4 * half + r % 4;
+            if (t < n && pc < vdim) y[(t0 + t) * inner + h * vdim + pc] = acc[r] + skip * x_s[t * 65 + 32 * pi + i];
+        }
+    }
+    // ---- U = B^T diag(w) X with w_s = exp(cum_last - cum_s) dt_s: tiles of 32 state rows by 32 columns
+    const float cum_last = cum_s[63];                        // (tokens beyond the block's add nothing to the sum)
+    float* dst = blocks > 1 ? block_states + (((int64_t)u * heads + h) * n_state) * vdim
+                            : state + (((int64_t)state_slots[s] * heads + h) * n_state) * vdim;
+    for (int tile = wave; tile < 2 * nt; tile += 4) {
+        const int ni = tile / 2, pi = tile % 2;
+        acc_t acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        const float* bcol = b_s + half * ld + 32 * ni + i;
+        const float* xcol = x_s + half * 65 + 32 * pi + i;
+#pragma unroll 8
+        for (int k = 0; k < 64; k += 2) {
+            const float w = expf(cum_last - cum_s[k + half]) * dt_s[k + half];
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(bcol[k * ld], w * xcol[k * 65], acc, 0, 0, 0);
+        }
+        const int pc = pw + 32 * pi + i;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = 32 * ni + 8 * (r / 4) + 4 * half + r % 4;
+            if (row < n_state && pc < vdim) dst[(int64_t)row * vdim + pc] = acc[r];
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------- what the state before a block adds
 // y[t, p] += exp(cum[t]) * sum_n C[t, n] E[n, p] for the tokens t of a block, E the true state before the block: one float
 // product per block and head, on the matrix cores (v_mfma_f32_32x32x2_f32: float operands, float sums).  A workgroup of
 // four waves takes 64 tokens of a block and 64 columns; C of those tokens and the 64 columns of E are staged in LDS (rows
 // beyond the state's are zero there).
-typedef __attribute__((ext_vector_type(16))) float ssd_f32x16;
 
 __global__ void __launch_bounds__(256)
 ssd_inter_kernel(const float* __restrict__ bc, int np, int heads, int vdim, int n_state, int groups,
@@ -473,12 +632,13 @@ static int ssd_padded_rows(int n_state) {
 NVA_EXPORT int NVA_NAME(nva_state_space_padded_rows)(int n_state) { return ssd_padded_rows(n_state); }
 
 template <int NPER, int NSPLIT>
-static void launch_scan(const ScanArgs& a, unsigned units, int first_seq, const int32_t* us, int mode, hipStream_t stream) {
+static void launch_scan(const ScanArgs& a, unsigned units, int first_seq, const int32_t* us, int mode, int carried_only,
+                        hipStream_t stream) {
     constexpr int PL = NVA_WAVE / NSPLIT;
     const dim3 grid((unsigned)((a.vdim + PL - 1) / PL), (unsigned)a.heads, units);
     hipLaunchKernelGGL((ssd_scan_kernel<elem_t, NPER, NSPLIT>), grid, dim3(NVA_WAVE), 0, stream, a.conv, a.channels, a.bc,
                        a.np, a.dtd, a.heads, a.vdim, a.n_state, a.groups, a.a_log, a.d_skip, a.state, a.cu, a.starts, a.slots,
-                       first_seq, us, mode, a.block_states, a.cum, a.y);
+                       first_seq, us, mode, carried_only, a.block_states, a.cum, a.y);
 }
 
 // proj: [tokens, 2 H P + 2 G N + H] with rows `stride` apart.  conv_out [tokens, C] (elements), y_raw [tokens, H P]
@@ -487,7 +647,8 @@ static void launch_scan(const ScanArgs& a, unsigned units, int first_seq, const 
 // portions of the requests from num_single on cut into blocks (units[u] = request counted from num_single, first token,
 // tokens, blocks of the portion; block_tokens: the most tokens of a block; shape: 0, or how a state of 65 to 128 rows is held (1: a thread a column, 2: four
 // lanes a column, 3: the second pass on the vector units, 4: single
-// tokens through the kernel that serves portions; measurements); chains[c] = first unit, blocks, request, tokens of the last block, for every
+// tokens through the kernel that serves portions, 6: blocks from a zero state
+// as products on the matrix cores; measurements); chains[c] = first unit, blocks, request, tokens of the last block, for every
 // portion of more than one block); null: every portion runs as one.
 // bc: float [tokens, groups, 2, padded rows] (zero where the padded rows exceed the state's: the caller clears it then),
 // dtd: float [tokens, heads, 2]: scratch as well.
@@ -532,14 +693,14 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
     const ScanArgs args{(const elem_t*)conv_out, channels, bc, ssd_padded_rows(n_state), dtd, heads, vdim, n_state, groups,
                         a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, block_states, cum, y_raw};
     // a thread holds up to 128 rows of a column of S; a state of more rows is shared out over 4 lanes
-    auto scan = [&](unsigned units, int first_seq, const int32_t* us, int mode) {
-        if (n_state <= 16) launch_scan<16, 1>(args, units, first_seq, us, mode, stream);
-        else if (n_state <= 32) launch_scan<32, 1>(args, units, first_seq, us, mode, stream);
-        else if (n_state <= 64) launch_scan<64, 1>(args, units, first_seq, us, mode, stream);
-        else if (n_state <= 128 && shape == 1) launch_scan<128, 1>(args, units, first_seq, us, mode, stream);
-        else if (n_state <= 128 && shape == 2) launch_scan<32, 4>(args, units, first_seq, us, mode, stream);
-        else if (n_state <= 128) launch_scan<64, 2>(args, units, first_seq, us, mode, stream);
-        else launch_scan<64, 4>(args, units, first_seq, us, mode, stream);
+    auto scan = [&](unsigned units, int first_seq, const int32_t* us, int mode, int carried_only = 0) {
+        if (n_state <= 16) launch_scan<16, 1>(args, units, first_seq, us, mode, carried_only, stream);
+        else if (n_state <= 32) launch_scan<32, 1>(args, units, first_seq, us, mode, carried_only, stream);
+        else if (n_state <= 64) launch_scan<64, 1>(args, units, first_seq, us, mode, carried_only, stream);
+        else if (n_state <= 128 && shape == 1) launch_scan<128, 1>(args, units, first_seq, us, mode, carried_only, stream);
+        else if (n_state <= 128 && shape == 2) launch_scan<32, 4>(args, units, first_seq, us, mode, carried_only, stream);
+        else if (n_state <= 128) launch_scan<64, 2>(args, units, first_seq, us, mode, carried_only, stream);
+        else launch_scan<64, 4>(args, units, first_seq, us, mode, carried_only, stream);
     };
     // the requests that bring one token (they come first) have a kernel of their own
     auto single = [&]() {
@@ -553,7 +714,26 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
     if (n_chains) {
         if (n_units <= 0 || n_units > 65535) return nva_fail("state_space: bad block count %lld", (long long)n_units);
         single();
-        scan((unsigned)n_units, (int)num_single, units, 1);
+        // blocks of up to 64 tokens from a zero state can run as three products on the matrix cores (shape 6; a portion's
+        // first block that goes on from the request's state, taller states and longer blocks run the recurrence): as
+        // fast as the recurrence where measured, and not the kernel that serves
+        const bool products = shape == 6 && block_tokens <= 64 && n_state <= 128;
+        if (products) {
+            const int nt = (n_state + 31) / 32;
+            const size_t lds = (size_t)(2 * 64 * (32 * nt + 1) + 2 * 64 * 65 + 128) * sizeof(float);
+            static bool raised_block = false;
+            if (!raised_block) {
+                if (hipFuncSetAttribute((const void*)ssd_block_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)((2 * 64 * 129 + 2 * 64 * 65 + 128) * sizeof(float))) != hipSuccess)
+                    return nva_fail("state_space: cannot have the LDS of the blocks' products");
+                raised_block = true;
+            }
+            hipLaunchKernelGGL(ssd_block_kernel, dim3((unsigned)((vdim + 63) / 64), (unsigned)heads, (unsigned)n_units), dim3(256),
+                               lds, stream, conv_out, (int)(sizeof(elem_t) == 4), channels, bc, ssd_padded_rows(n_state), dtd,
+                               heads, vdim, n_state, groups, a_log, d_skip, state, cu_seqlens, seq_starts, state_slots,
+                               (int)num_single, units, block_states, cum, y_raw);
+        }
+        scan((unsigned)n_units, (int)num_single, units, 1, products ? 1 : 0);
         hipLaunchKernelGGL(ssd_chain_kernel, dim3((n_state * vdim + 255) / 256, heads, (unsigned)n_chains), dim3(256), 0, stream,
                            block_states, cum, state, chains, units, cu_seqlens, state_slots, (int)num_single, heads, n_state,
                            vdim);

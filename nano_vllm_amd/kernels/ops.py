@@ -150,6 +150,25 @@ def retention_blocks(q_lens, first_seq: int):
     return bt, units, chains
 
 
+def state_space_blocks(q_lens, first_seq: int):
+    """As retention_blocks, for the state-space layer's blocks as products: blocks of 64 tokens, which that kernel takes, as long
+    as the step's portions hold at most 16384 tokens (a block's end state is kept until the pass over the blocks);
+    beyond that the blocks double as retention's do."""
+    total = sum(q_lens[first_seq:])
+    if total > 16384:
+        return retention_blocks(q_lens, first_seq)
+    bt = 64
+    units, chains = [], []
+    for s in range(first_seq, len(q_lens)):
+        n = q_lens[s]
+        nb = (n + bt - 1) // bt
+        if nb > 1:
+            chains += [len(units) // 4, nb, s - first_seq, n - (nb - 1) * bt]
+        for b in range(nb):
+            units += [s - first_seq, b * bt, min(bt, n - b * bt), nb]
+    return bt, units, chains
+
+
 def prefill_tile_order(q_lens, starts, first_seq: int) -> list:
     """Flat [(request, row tile), ...] of the requests from `first_seq` on, from the tile that
     sees the most keys to the one that sees the fewest: the prefill attention kernel hands its
@@ -285,7 +304,8 @@ class HipKernels:
         # False: the state-space layer runs a portion's tokens one after the other, whatever its length
         self.state_space_blocks_side_by_side = True
         # how the recurrence holds a state of 65 to 128 rows: 0 two lanes a column (what serves), 1 a thread a column
-        # with scalar operands, 2 four lanes a column (measurements)
+        # with scalar operands, 2 four lanes a column, 3 the second pass of the blocks on the vector units, 4 single
+        # tokens through the kernel of the portions, 6 blocks from a zero state as products on the matrix cores (measurements)
         self.state_space_shape = 0
 
     # ------------------------------------------------------------------ helpers
@@ -1278,16 +1298,17 @@ class HipKernels:
             kept = getattr(batch, "step_cache", None)
             if kept is None:
                 kept = batch.step_cache = {}
-            plan = kept.get(("state_space_blocks", first))
+            plan = kept.get(("state_space_blocks", first, self.state_space_shape == 6))
             if plan is None:
-                block_tokens, flat_units, flat_chains = retention_blocks(batch.q_lens, first)
+                block_tokens, flat_units, flat_chains = (state_space_blocks if self.state_space_shape == 6 else retention_blocks)(
+                    batch.q_lens, first)
                 if flat_chains:
                     both = torch.tensor(flat_units + flat_chains, dtype=torch.int32).to(proj.device, non_blocking=True)
                     plan = (len(flat_units) // 4, len(flat_chains) // 4, both[: len(flat_units)], both[len(flat_units):],
                             block_tokens)
                 else:
                     plan = (0, 0, None, None, 0)
-                kept[("state_space_blocks", first)] = plan
+                kept[("state_space_blocks", first, self.state_space_shape == 6)] = plan
             n_units, n_chains, units, chains, block_tokens = plan
             if n_chains:
                 block_states = torch.empty((n_units, heads, n_state, vdim), dtype=torch.float32, device=proj.device)

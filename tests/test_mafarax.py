@@ -423,6 +423,16 @@ def test_state_space_of_long_portions_whose_blocks_run_side_by_side(dtype):
     _close(got, one.cpu(), dtype, "one after the other", tol=1e-2 if dtype == torch.bfloat16 else 2e-4)
     for a, b in zip(kept, states):
         _close(a, b.cpu(), torch.float32, "the states left behind", tol=2e-4)
+    # the blocks from a zero state as products on the matrix cores: the same outputs and states
+    k.state_space_shape = 6
+    try:
+        states = _new_states(dev, 5, shape, fill=float("nan"))
+        prod = _run_ssm(k, dev, torch.cat(projs), w, shape, 1e-6, states, lens, [0] * 5, [0, 1, 2, 3, 4])
+    finally:
+        k.state_space_shape = 0
+    _close(got, prod.cpu(), dtype, "as products", tol=1e-2 if dtype == torch.bfloat16 else 2e-4)
+    for a, b in zip(kept, states):
+        _close(a, b.cpu(), torch.float32, "the states the products left", tol=2e-4)
     # and the next portion goes on from the state the blocks left
     more = (torch.randn((40, width), generator=g)).to(dtype)
     both = _plain_ssm_of_projections(torch.cat((projs[1], more)), w, heads, vdim, n_state, groups, norm_groups, 1e-6)[700:]
