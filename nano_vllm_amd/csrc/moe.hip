@@ -8,15 +8,16 @@
 //             their experts the `top` with the largest scores are chosen (equal scores: the lower number);
 //             ids [tokens, top], weights [tokens, top] = scale * s.
 //   plan      the pairs (token, choice) counted and sorted by expert: place[pair] = the pair's row among the
-//             sorted ones, rows[place] = pair; the sorted rows cut into tiles of MOE_BM rows of one expert:
+//             sorted ones, rows[place] = pair; the sorted rows cut into tiles of 32 or 128 rows of one expert:
 //             tile_expert[i], tile_row0[i], tile_rows[i], and their number.
-//   up        h[row] = act(x[token of row] Wu_e^T)         rows sorted by expert, a tile of rows and 64 outputs
-//   down      o[row] = h[row] Wd_e^T                       to a workgroup
+//   up        h[row] = act(x[token of row] Wu_e^T)         rows sorted by expert, a tile of rows and 64 or 128
+//   down      o[row] = h[row] Wd_e^T                       outputs to a workgroup
 //   combine   y[token] = sum over its choices of weight * o[place] (+ add[token])
 //
-// The products are float sums over k in ascending order, one chain per output, so a token's result does
-// not depend on what else is in the batch or on where its row fell among the sorted ones; operands and
-// results are elements (rounded once), the combination is float.
+// The products are float sums of a row by itself (on the vector units over k in ascending order, one chain per
+// output; on the matrix cores in the order of the instruction's steps), so a token's result does not depend on
+// what else is in the batch or on where its row fell among the sorted ones; operands and results are elements
+// (rounded once), the combination is float.
 #include "common.h"
 
 #define MOE_BM 32

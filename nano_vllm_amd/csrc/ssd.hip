@@ -15,13 +15,16 @@
 // (step sizes, decays, the state, the read-out, gate and norm) is float with the accurate exponential
 // and logarithm in both builds, rounded once at the output.
 //
-// Kernels: conv (a thread per token and channel; a request that brings one token also shifts its kept
-// inputs), conv_state (the kept inputs of requests that bring a portion), scan, finish.  The scan gives
-// every thread one column of S (up to 64 of its rows, in registers: a state of more rows is shared out over
-// 2 or 4 lanes, whose sums meet by shuffles); B, C and x of 16 tokens at a time are staged in LDS for the wave.  A long portion is cut into blocks that
+// Kernels: conv (a thread per token and channel, or eight tokens in a row; it also leaves B and C as floats
+// and every head's step size and decay; a request that brings one token shifts its kept inputs there),
+// conv_state (the kept inputs of requests that bring a portion), single (requests that bring one token),
+// scan (portions), chain and inter (blocks), finish.  The scan gives every thread one column of S (up to 64 of
+// its rows, in registers: a state of more rows is shared out over 2 or 4 lanes, whose sums meet by shuffles);
+// B, C and x of 16 tokens at a time are staged in LDS for the wave.  A long portion is cut into blocks that
 // run side by side, each from a zero state (the first from the request's); a pass over the blocks makes
 // every block's true state at its end, E_b = exp(sum of the block's log-decays) E_(b-1) + U_b, and a
-// second pass adds what the state before a block contributes, exp(log-decay up to t) E_(b-1)^T C_t.
+// second pass, a float product on the matrix cores, adds what the state before a block contributes,
+// exp(log-decay up to t) E_(b-1)^T C_t.
 #include "common.h"
 
 #define SSD_MAX_TAPS 16
@@ -137,7 +140,7 @@ ssd_conv_state_kernel(const T* __restrict__ proj, int64_t stride, int col0, int 
 // mode 2 (blocks, second pass): the blocks after a portion's first add exp(cum_t) E^T C_t to y, E the true
 //         state before the block (block_states[u - 1] after the pass over the blocks).
 // B, C, the step size and the decay of a token are the same for all lanes of a wave.  Where a thread holds a whole
-// column of S (NSPLIT 1: up to 128 rows) they are read from global memory by addresses that are the same in
+// column of S (NSPLIT 1: up to 64 rows, or 128 where asked for) they are read from global memory by addresses that are the same in
 // every lane, which the compiler turns into scalar loads: they cost no vector register and no LDS, and are
 // operands of the multiply-adds as they are.  Where a column is shared out over lanes, B and C of 16 tokens at a
 // time go through LDS.
@@ -692,7 +695,7 @@ NVA_EXPORT int NVA_NAME(nva_state_space)(const void* proj, int64_t stride, void*
                            state_slots, (int)num_single);
     const ScanArgs args{(const elem_t*)conv_out, channels, bc, ssd_padded_rows(n_state), dtd, heads, vdim, n_state, groups,
                         a_log, d_skip, state, cu_seqlens, seq_starts, state_slots, block_states, cum, y_raw};
-    // a thread holds up to 128 rows of a column of S; a state of more rows is shared out over 4 lanes
+    // a thread holds up to 64 rows of a column of S; a state of more rows is shared out over 2 or 4 lanes
     auto scan = [&](unsigned units, int first_seq, const int32_t* us, int mode, int carried_only = 0) {
         if (n_state <= 16) launch_scan<16, 1>(args, units, first_seq, us, mode, carried_only, stream);
         else if (n_state <= 32) launch_scan<32, 1>(args, units, first_seq, us, mode, carried_only, stream);
