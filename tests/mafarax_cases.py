@@ -58,6 +58,21 @@ CONFIGS: Dict[str, dict] = {
                      Ssm(heads=6, vdim=12, state=16, groups=3, conv=4, norm_groups=2),
                      Moe(experts=15, top=2, ff=30, scale=1.0, group_count=5, group_keep=2, shared_ff=30)),)),
         page=16, seed=34),
+    # a larger one for long prompts: six layers, three chunk sizes (three cache groups), a layer without rotation, one
+    # without feed-forward, key/value heads as many as query heads and one for all, convolutions of 2 to 5 taps
+    "e": dict(cfg=MafaraxConfig(vocab=384, width=320, eps=1e-5, logit_scale=0.7, layers=(
+        MafaraxLayer(Att(5, 5, 64, 48, 0.11, 160, rot_dims=32, rot_base=2e4, rot_factor=1.0),
+                     Ssm(heads=8, vdim=40, state=48, groups=2, conv=3, norm_groups=2),
+                     Moe(experts=10, top=3, ff=72, scale=0.8, group_count=5, group_keep=2, shared_ff=128)),
+        MafaraxLayer(Att(5, 1, 64, 48, 0.11, 160, rot_dims=32, rot_base=2e4, rot_factor=1.0),
+                     Ssm(heads=8, vdim=40, state=48, groups=2, conv=3, norm_groups=2), None),
+        MafaraxLayer(Att(5, 5, 64, 48, 0.11, 70),
+                     Ssm(heads=8, vdim=40, state=48, groups=4, conv=5, norm_groups=1),
+                     Moe(experts=10, top=3, ff=72, scale=0.8, group_count=5, group_keep=2, shared_ff=128)),
+        MafaraxLayer(Att(5, 5, 64, 48, 0.11, 1000, rot_dims=32, rot_base=2e4, rot_factor=1.0),
+                     Ssm(heads=8, vdim=40, state=48, groups=1, conv=2, norm_groups=4),
+                     Moe(experts=10, top=3, ff=72, scale=0.8, group_count=5, group_keep=2, shared_ff=128)))),
+        page=64, seed=35),
 }
 
 _folders: Dict[str, str] = {}

@@ -578,6 +578,22 @@ def test_bfloat16_follows_the_plain_logits_under_every_cutting(name):
             and float(e.max()) < 0.6, (portions, float(e.median()), float(e.max()))
 
 
+@pytest.mark.gpu
+def test_a_larger_model_over_long_prompts():
+    """Six hundred tokens through a model of three cache groups: whole (the recurrence in blocks side by side, keys
+    hundreds of positions back inside the longest chunk), in changing portions, and its last tokens one by one."""
+    name = "e"
+    c = M.CONFIGS[name]
+    n = 600
+    toks = H.random_tokens(c["cfg"].vocab, n, 17)
+    want = M.plain_logits(M.model_folder(name), toks)
+    r = _runner(name, "hip", "float32", 12)
+    assert len(r.cache.groups) == 3
+    for portions in (H.whole(n), H.changing_portions(n, 5), H.last_one_by_one(n, 70)):
+        assert M.err(H.run_portions(r, "x", toks, portions), want) < MODEL_TOL["float32"], portions[:4]
+    assert all(pool.num_free == 12 for pool in r.cache.pools)
+
+
 @pytest.mark.parametrize("backend", BACKENDS)
 def test_the_first_tokens_of_a_sequence(backend):
     for name in ("a", "c"):
